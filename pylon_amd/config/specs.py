@@ -89,7 +89,14 @@ class SinkAttentionSpec:
     denominator).  ``score = scale * q.k + rel[bucket(i - j), head]`` with ``bias_rows`` rows in
     ``rel``: distances below ``bias_rows // 2`` have a row each, the other half of the rows
     spreads logarithmically up to ``bias_far``, beyond which the last row is used.  Keys have
-    ``head_dim`` elements, values ``v_head_dim``."""
+    ``head_dim`` elements, values ``v_head_dim``.
+
+    ``bias_form="log"`` replaces the table by two learned numbers per head, ``a`` and ``b``:
+    ``score = scale * q.k - a * log(1 + b * (i - j))`` (``bias_rows`` and ``bias_far`` are then
+    unused).  ``chunk``: position ``i`` sees key ``j <= i`` only inside its own chunk of that many
+    positions (as in :class:`AttentionSpec`; not together with a window).  ``qkv_bias``: the q, k and v
+    projections have a bias each.  ``own_kv`` False: a layer that only ever runs on another run's keys
+    and values and has no k and v projections of its own."""
 
     hidden_size: int
     n_heads: int
@@ -102,6 +109,13 @@ class SinkAttentionSpec:
     sink: bool = True
     window: Optional[int] = None
     kind: str = "sink_attention"
+    bias_form: str = "table"
+    chunk: Optional[int] = None
+    qkv_bias: bool = False
+    own_kv: bool = True
+    # False: the cache keeps every token's keys and values although the layer's own mask would let
+    # old pages go (runs with other masks read the same cache)
+    cache_bounded: bool = True
 
 
 @dataclass(frozen=True)
@@ -148,6 +162,26 @@ class RetentionSpec:
 
 
 @dataclass(frozen=True)
+class TokenShiftSpec:
+    """``h + (h' - h) * w``: every token's input moved towards the previous token's (``h'``, zeros
+    before a request's first token) by a learned share per channel; a request's last input is its
+    state."""
+
+    dim: int
+    kind: str = "token_shift"
+
+
+@dataclass(frozen=True)
+class SinusoidPositionSpec:
+    """A fixed position vector added to the embedded tokens: element ``2i`` is
+    ``sin(p * base**(-2i/dim))``, element ``2i + 1`` the cosine of the same angle."""
+
+    dim: int
+    base: float = 10000.0
+    kind: str = "sinusoid"
+
+
+@dataclass(frozen=True)
 class ShortConvSpec:
     """``h + conv(h)``: a causal convolution of ``taps`` taps over time on each of ``dim``
     channels, added to its input; a request's last ``taps - 1`` inputs are its state."""
@@ -176,7 +210,15 @@ class MixtureFeedForwardSpec:
     every token uses the ``top`` with the largest router logits ``W_r h + b`` (float32), weighted
     by the softmax over those ``top`` logits alone; an expert is ``down(silu(gate(h)) * up(h))``.
     With ``shared_size`` a further expert of that many hidden units runs for every token and is
-    added, multiplied by ``sigmoid(w_sg . h)`` if ``shared_gate``."""
+    added, multiplied by ``sigmoid(w_sg . h)`` if ``shared_gate``.
+
+    ``expert_act="relu2"``: plain experts, ``down(relu(up(h))^2)``.  ``scoring="softmax_all"``: the
+    scores are the softmax over all router outputs; the ``router_bias`` is a correction added to
+    them for the choice only; the router's outputs form ``groups`` equal groups of neighbours of
+    which only the ``groups_kept`` with the largest corrected score can be chosen from; the weights
+    are the chosen scores times ``route_scale``, not renormalised.  The router's last ``n_identity``
+    outputs (beyond the ``n_experts`` experts, and counted in the groups) are identity experts whose
+    output is the input itself."""
 
     hidden_size: int
     n_experts: int
@@ -186,6 +228,12 @@ class MixtureFeedForwardSpec:
     shared_gate: bool = True
     router_bias: bool = True
     kind: str = "mixture"
+    expert_act: str = "silu_gated"
+    scoring: str = "top_softmax"
+    n_identity: int = 0
+    groups: int = 1
+    groups_kept: int = 1
+    route_scale: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -206,12 +254,14 @@ class LogitScaleSpec:
 
 @dataclass(frozen=True)
 class GatedFeedForwardSpec:
-    """``down(act(gate(x)) * up(x))`` with gate and up fused into one matrix."""
+    """``down(act(gate(x)) * up(x))`` with gate and up fused into one matrix; with ``bias`` all
+    three projections have one."""
 
     hidden_size: int
     intermediate_size: int
     activation: str = "silu"
     kind: str = "gated_mlp"
+    bias: bool = False
 
 
 @dataclass(frozen=True)
@@ -222,6 +272,12 @@ class LayerSpec:
     ``arrangement="sandwich_norm"``: every sublayer is normed on both sides,
     ``x += post1(mixer(conv(norm1(x)))); x += post2(ff(norm2(x)))``, where ``conv`` is the
     optional ``input_conv`` in front of the mixer and ``feed_forward`` may be None.
+
+    In the ``pre_norm`` arrangement: ``input_conv`` (a short convolution or a token shift) works on
+    ``norm1``'s output; with ``sublayer_scale`` each sublayer's output is multiplied element by element
+    by a learned vector before it is added; ``depth_mix = (index, total)`` makes the layer's result
+    stream ``index`` of ``total`` (stream 0: the embedded tokens) and hands on, instead of it, a learned
+    mix ``sum_{j <= index} c[j] * stream_j`` of all streams so far.
     """
 
     mixer: object
@@ -232,6 +288,8 @@ class LayerSpec:
     mixer_post_norm: Optional[NormSpec] = None
     feed_forward_post_norm: Optional[NormSpec] = None
     input_conv: Optional[object] = None
+    sublayer_scale: bool = False
+    depth_mix: Optional[Tuple[int, int]] = None
 
     @property
     def kind(self) -> str:

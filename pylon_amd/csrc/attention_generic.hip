@@ -7,8 +7,10 @@
 // of every sum depends only on the token's position and never on how the batch was cut.
 // Options: values of another size than keys; q rows that lie q_stride elements apart (a slice
 // of a fused projection); a learned bias by distance added to the scaled score,
-// rel[bucket[min(i - j, bucket_len - 1)] * n_heads + head]; and a sink, a key of score 0
-// without a value, which adds one to the softmax's denominator.
+// rel[bucket[min(i - j, bucket_len - 1)] * n_heads + head], or without a table of buckets a bias
+// that grows with the logarithm of the distance and is taken off, rel[head] * log(1 + rel[n_heads +
+// head] * (i - j)); and a sink, a key of score 0 without a value, which adds one to the softmax's
+// denominator.
 #include "common.h"
 
 #define ATT_WAVES 4
@@ -99,7 +101,10 @@ __global__ void paged_attention_kernel(T* __restrict__ out, const T* __restrict_
       s = dot * scale;
       if (rel != nullptr) {
         const int far = pos - j;
-        s += rel[static_cast<size_t>(bucket[far < bucket_len ? far : bucket_len - 1]) * n_heads + h];
+        if (bucket != nullptr)
+          s += rel[static_cast<size_t>(bucket[far < bucket_len ? far : bucket_len - 1]) * n_heads + h];
+        else
+          s -= rel[h] * logf(1.0f + rel[n_heads + h] * static_cast<float>(far));
       }
     }
     const float m_new = fmaxf(m, wave_max(s));
@@ -167,7 +172,8 @@ static int launch_paged_attention(T* out, const T* q, const T* k_cache, const T*
 // q: [tokens, n_heads, head_dim], rows q_stride elements apart; out: [tokens, n_heads, v_dim].
 // Caches: keys [pages*page_size, n_kv_heads, head_dim], values [pages*page_size, n_kv_heads, v_dim].
 // With v_transposed the values lie as [pages, n_kv_heads, v_dim, page_size].
-// rel: null, or float [rows, n_heads] with bucket: int [bucket_len], every entry a row of rel.
+// rel: null, or float [rows, n_heads] with bucket: int [bucket_len], every entry a row of rel; or,
+// with bucket null, float [2, n_heads]: per head the factor and the slope of a logarithmic bias.
 // block_table: [rows, table_width] page ids; tok_row[t] names the table row of token t;
 // positions[t] is the token's index in its request; keys first(t)..positions[t] are read,
 // first(t) = max(0, positions[t] - window + 1) when window > 0; the start of the token's chunk of
@@ -187,8 +193,8 @@ extern "C" int pylon_paged_attention(void* out, const void* q, const void* k_cac
   PYLON_REQUIRE(page_size > 0 && table_width > 0, "paged_attention: bad page size or table width");
   PYLON_REQUIRE(v_dim >= 1 && v_dim <= 512, "paged_attention: values of 1 to 512 elements, got %d", v_dim);
   PYLON_REQUIRE(q_stride >= static_cast<long long>(n_heads) * head_dim, "paged_attention: q rows overlap");
-  PYLON_REQUIRE(rel == nullptr || (bucket != nullptr && bucket_len >= 1),
-                "paged_attention: a bias by distance needs its table of buckets");
+  PYLON_REQUIRE(rel == nullptr || bucket == nullptr || bucket_len >= 1,
+                "paged_attention: a table of buckets holds at least one entry");
   if (tokens == 0) return 0;
   PYLON_REQUIRE(static_cast<long long>(tokens) * n_heads / ATT_WAVES < (1ll << 31),
                 "paged_attention: too many (token, head) pairs for one launch");

@@ -44,7 +44,7 @@ __global__ __launch_bounds__(512) void attention_sink_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, const int* __restrict__ positions, int n_heads, int n_kv_heads, int dim, int vdim, int page_size, float scale,
-    const float* __restrict__ bias, int bucket_len, int sink, int cuts, float* __restrict__ partial) {
+    const float* __restrict__ bias, int bucket_len, int sink, int cuts, float* __restrict__ partial, int window) {
   // eight waves: wave & 3 names the head of the group, wave >> 2 which 16 of the tile's 32 tokens, so
   // that every SIMD holds two waves that fill each other's waits
   constexpr int waves_per_group = 4;
@@ -87,11 +87,12 @@ __global__ __launch_bounds__(512) void attention_sink_kernel(
 
   // Q^T operands: column = query, eight key elements per lane and step
   bf16x8 qf[AS_QT][KS];
-  int qpos[AS_QT];
+  int qpos[AS_QT], qfirst[AS_QT];  // a query's position and the first key it sees (a window, a chunk)
 #pragma unroll
   for (int qt = 0; qt < AS_QT; ++qt) {
     const int qi = (qt + qsel) * 16 + col;
     qpos[qt] = pos0 + qi;
+    qfirst[qt] = first_visible(qpos[qt], window);
     const int t = tok0 + (qi < count ? qi : count - 1);
     const bf16_t* qr = q + static_cast<size_t>(t) * q_stride + static_cast<size_t>(head) * dim;
 #pragma unroll
@@ -114,10 +115,12 @@ __global__ __launch_bounds__(512) void attention_sink_kernel(
     for (int dt = 0; dt < NV; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  const int n_blocks = kv_last / AS_BLOCK + 1;
+  // the walk starts at the block of the first key that the tile's first query sees
+  const int kb_first = first_visible(pos0, window) / AS_BLOCK * AS_BLOCK;
+  const int n_blocks = (kv_last - kb_first) / AS_BLOCK + 1;
   const int per_cut = (n_blocks + cuts - 1) / cuts;
-  const int kb_begin = cut * per_cut * AS_BLOCK;
-  const int kb_end = (cut + 1) * per_cut < n_blocks ? (cut + 1) * per_cut * AS_BLOCK : n_blocks * AS_BLOCK;
+  const int kb_begin = kb_first + cut * per_cut * AS_BLOCK;
+  const int kb_end = kb_first + ((cut + 1) * per_cut < n_blocks ? (cut + 1) * per_cut : n_blocks) * AS_BLOCK;
   // A block's keys and values travel global -> registers -> LDS; the registers of block b + 1
   // are filled while block b is computed.
   u32x4 kreg[KL], vreg[VL];
@@ -237,7 +240,7 @@ __global__ __launch_bounds__(512) void attention_sink_kernel(
           bias = tbl[idx];
         }
         const float v = fmaf(s[qt][e >> 2][e & 3], scale, bias);
-        sc[e] = dist >= 0 ? v : -INFINITY;
+        sc[e] = (dist >= 0 && key >= qfirst[qt]) ? v : -INFINITY;
         top = fmaxf(top, sc[e]);
       }
       top = fmaxf(top, __shfl_xor(top, 16, 64));
@@ -332,7 +335,7 @@ __global__ __launch_bounds__(256) void attention_sink_decode_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ positions, int n_heads, int n_kv_heads, int dim, int vdim, int page_size, float scale,
-    const float* __restrict__ bias, int bucket_len, int sink, int cuts, float* __restrict__ partial) {
+    const float* __restrict__ bias, int bucket_len, int sink, int cuts, float* __restrict__ partial, int window) {
   extern __shared__ float bias_lds[];  // [group][bucket_len]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
@@ -373,10 +376,12 @@ __global__ __launch_bounds__(256) void attention_sink_decode_kernel(
   float m_run = first ? 0.f : -INFINITY;
   float l_run = (first && grp == 0) ? 1.f : 0.f;
 
-  const int n_blocks = pos / AS_BLOCK + 1;
+  const int first_key = first_visible(pos, window);  // a window, a chunk: the walk starts at its block
+  const int kb_first = first_key / AS_BLOCK * AS_BLOCK;
+  const int n_blocks = (pos - kb_first) / AS_BLOCK + 1;
   const int per_cut = (n_blocks + cuts - 1) / cuts;
-  const int kb_begin = cut * per_cut * AS_BLOCK;
-  const int kb_end = (cut + 1) * per_cut < n_blocks ? (cut + 1) * per_cut * AS_BLOCK : n_blocks * AS_BLOCK;
+  const int kb_begin = kb_first + cut * per_cut * AS_BLOCK;
+  const int kb_end = kb_first + ((cut + 1) * per_cut < n_blocks ? (cut + 1) * per_cut : n_blocks) * AS_BLOCK;
   for (int kb = kb_begin + wave * AS_BLOCK; kb < kb_end; kb += 4 * AS_BLOCK) {
     const int page = table[kb / page_size];
     const int in_page = kb % page_size;
@@ -430,7 +435,7 @@ __global__ __launch_bounds__(256) void attention_sink_decode_kernel(
         add = tbl[idx];
       }
       const float v = fmaf(s[e >> 2][e & 3], scale, add);
-      sc[e] = dist >= 0 ? v : -INFINITY;
+      sc[e] = (dist >= 0 && key >= first_key) ? v : -INFINITY;
       top = fmaxf(top, sc[e]);
     }
     top = fmaxf(top, __shfl_xor(top, 16, 64));
@@ -537,12 +542,13 @@ __global__ void attention_sink_merge_kernel(bf16_t* __restrict__ out, const floa
 // consecutive tokens of one request; or null, and then positions: int [n_tiles], one token per tile,
 // token t on row t of the block table (a step of single tokens).  bias: null or float [n_heads, bucket_len
 // <= 4096], a head's bias by distance, the last entry for every distance from bucket_len - 1 on.  dim a multiple of 8 up to 256, vdim a multiple of 4
-// up to 256, page_size a multiple of 32.  The host guarantees that the tiles lie inside q and the table.
+// up to 256, page_size a multiple of 32.  window: the mask as one integer (first_visible in common.h).
+// The host guarantees that the tiles lie inside q and the table.
 extern "C" int pylon_attention_sink(void* out, const void* q, long long q_stride, const void* k_cache,
                                     const void* v_cache, const int* block_table, int table_width, const int* tiles,
                                     const int* positions, int n_tiles, int n_heads, int n_kv_heads, int dim, int vdim, int page_size,
                                     float scale, const float* bias, int bucket_len, int sink,
-                                    int cuts, float* partial, long long partial_floats, int tokens,
+                                    int cuts, float* partial, long long partial_floats, int tokens, int window,
                                     hipStream_t stream) {
   PYLON_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                 "attention_sink: %d query heads cannot be grouped over %d key/value heads", n_heads, n_kv_heads);
@@ -582,7 +588,7 @@ extern "C" int pylon_attention_sink(void* out, const void* q, long long q_stride
     hipLaunchKernelGGL((attention_sink_decode_kernel<KS, NV>), dim3(static_cast<unsigned>(wgs)), dim3(256), lds_d,    \
                        stream, (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,           \
                        block_table, table_width, positions, n_heads, n_kv_heads, dim, vdim, page_size, scale, bias,  \
-                       bias != nullptr ? bucket_len : 1, sink, cuts, partial);                                       \
+                       bias != nullptr ? bucket_len : 1, sink, cuts, partial, window);                               \
   } while (0)
 #define PICK_D(KS)                  \
   do {                              \
@@ -622,7 +628,7 @@ extern "C" int pylon_attention_sink(void* out, const void* q, long long q_stride
                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
   hipLaunchKernelGGL((attention_sink_kernel<KS, NV>), grid, block, lds, stream, (bf16_t*)out, (const bf16_t*)q, \
                      q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, tiles, \
-                     positions, n_heads, n_kv_heads, dim, vdim, page_size, scale, bias, table_len, sink, cuts, partial); \
+                     positions, n_heads, n_kv_heads, dim, vdim, page_size, scale, bias, table_len, sink, cuts, partial, window); \
   } while (0)
 #define PICK_NV(KS)                 \
   do {                              \

@@ -417,7 +417,7 @@ extern "C" int pylon_silu_gate(void* out, int out_dtype, const void* gate_up, in
 // the linear branch and cap are the caller's (limit <= 0: no cap).
 template <typename TI, typename TO>
 __global__ void gated_act_kernel(TO* __restrict__ out, const TI* __restrict__ gu, int inter, size_t total,
-                                 float alpha, float offset, float limit) {
+                                 float alpha, float offset, float limit, const float* __restrict__ bias) {
   size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
   for (; i < total; i += step) {
@@ -425,6 +425,10 @@ __global__ void gated_act_kernel(TO* __restrict__ out, const TI* __restrict__ gu
     const size_t c = i - t * inter;
     float g = to_float(gu[t * 2 * inter + c]);
     float u = to_float(gu[t * 2 * inter + inter + c]);
+    if (bias != nullptr) {  // the two projections' biases, [2 inter]
+      g += bias[c];
+      u += bias[inter + c];
+    }
     if (limit > 0.f) {
       g = fminf(g, limit);
       u = fminf(fmaxf(u, -limit), limit);
@@ -465,12 +469,12 @@ __global__ void gated_act_bf16x8_kernel(uint4* __restrict__ out, const uint4* __
 }
 
 extern "C" int pylon_gated_act(void* out, int out_dtype, const void* gate_up, int in_dtype, int tokens, int inter,
-                               float alpha, float offset, float limit, hipStream_t stream) {
+                               float alpha, float offset, float limit, const float* bias, hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(in_dtype) && pylon_valid_dtype(out_dtype), "gated_act: unknown dtype");
   PYLON_REQUIRE(tokens >= 0 && inter > 0, "gated_act: bad sizes tokens=%d inter=%d", tokens, inter);
   const size_t total = static_cast<size_t>(tokens) * inter;
   if (total == 0) return 0;
-  if (in_dtype == PYLON_BF16 && out_dtype == PYLON_BF16 && inter % 8 == 0 &&
+  if (bias == nullptr && in_dtype == PYLON_BF16 && out_dtype == PYLON_BF16 && inter % 8 == 0 &&
       (reinterpret_cast<uintptr_t>(out) & 15) == 0 && (reinterpret_cast<uintptr_t>(gate_up) & 15) == 0) {
     const size_t chunks_total = total / 8;
     size_t nblocks = (chunks_total + 255) / 256;
@@ -484,7 +488,7 @@ extern "C" int pylon_gated_act(void* out, int out_dtype, const void* gate_up, in
   dim3 grid((unsigned)blocks), block(256);
 #define GO(TI, TO)                                                                                             \
   hipLaunchKernelGGL((gated_act_kernel<TI, TO>), grid, block, 0, stream, (TO*)out, (const TI*)gate_up, inter, \
-                     total, alpha, offset, limit)
+                     total, alpha, offset, limit, bias)
   if (in_dtype == PYLON_F32 && out_dtype == PYLON_F32) GO(float, float);
   else if (in_dtype == PYLON_F32) GO(float, bf16_t);
   else if (out_dtype == PYLON_F32) GO(bf16_t, float);
@@ -524,4 +528,58 @@ extern "C" int pylon_softcap(float* x, long long count, float cap, hipStream_t s
   if (blocks > 65535u * 16u) blocks = 65535u * 16u;
   hipLaunchKernelGGL(softcap_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, (size_t)count, cap);
   PYLON_LAUNCHED("softcap");
+}
+
+// ---- sinusoidal positions ----------------------------------------------------------------------
+// x[t, 2i] += sin(p_t * f_i), x[t, 2i + 1] += cos(p_t * f_i): the angle is the float product of the
+// token's position and a frequency that the caller formed once; sine and cosine with full range
+// reduction.
+__global__ void add_sinusoid_kernel(float* __restrict__ x, const int* __restrict__ positions,
+                                    const float* __restrict__ freq, int dim, size_t total_pairs, int pairs) {
+  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (; i < total_pairs; i += step) {
+    const size_t t = i / pairs;
+    const int k = static_cast<int>(i - t * pairs);
+    const float angle = static_cast<float>(positions[t]) * freq[k];
+    float* row = x + t * dim;
+    row[2 * k] += sinf(angle);
+    if (2 * k + 1 < dim) row[2 * k + 1] += cosf(angle);
+  }
+}
+
+// x: float [tokens, dim]; positions: int [tokens]; freq: float [(dim + 1) / 2].
+extern "C" int pylon_add_sinusoid(float* x, const int* positions, const float* freq, int tokens, int dim,
+                                  hipStream_t stream) {
+  PYLON_REQUIRE(tokens >= 0 && dim > 0, "add_sinusoid: bad sizes");
+  if (tokens == 0) return 0;
+  const int pairs = (dim + 1) / 2;
+  const size_t total = static_cast<size_t>(tokens) * pairs;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65535u * 16u) blocks = 65535u * 16u;
+  hipLaunchKernelGGL(add_sinusoid_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, positions, freq, dim, total,
+                     pairs);
+  PYLON_LAUNCHED("add_sinusoid");
+}
+
+// ---- a bias per column, in place -----------------------------------------------------------------
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ x, const float* __restrict__ bias, int dim, size_t total) {
+  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (; i < total; i += step) x[i] = from_float<T>(to_float(x[i]) + bias[i % dim]);
+}
+
+// x: [rows, dim] of dtype, contiguous; bias: float [dim].
+extern "C" int pylon_add_bias(void* x, int dtype, const float* bias, long long rows, int dim, hipStream_t stream) {
+  PYLON_REQUIRE(pylon_valid_dtype(dtype) && rows >= 0 && dim > 0, "add_bias: bad arguments");
+  const size_t total = static_cast<size_t>(rows) * dim;
+  if (total == 0) return 0;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65535u * 16u) blocks = 65535u * 16u;
+  if (dtype == PYLON_F32)
+    hipLaunchKernelGGL(add_bias_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, (float*)x, bias, dim, total);
+  else
+    hipLaunchKernelGGL(add_bias_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, (bf16_t*)x, bias, dim, total);
+  PYLON_LAUNCHED("add_bias");
 }

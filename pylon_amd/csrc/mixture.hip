@@ -8,6 +8,13 @@
 //   its chosen experts e = experts[t, s]; a workgroup takes one (token, choice) and some hidden
 //   units, the token's input in LDS, a wave a hidden unit at a time with the lanes along the row.
 // expert_down: out[t] = sum_s weight[t, s] W_down[e_s] hidden[(t, s)] (+ gate[t] * shared[t]), float.
+// route_scored: the other way to choose: scores are the softmax over all router outputs; a
+//   correction is added to them for the choice only; the outputs form equal groups of neighbours of
+//   which only the best few (by their largest corrected score) may be chosen from; the weights are the
+//   chosen scores times a constant, not renormalised.  The last router outputs may be identity
+//   experts, whose output is the token's input itself: their weights are summed into one number per
+//   token, and the expert kernels pass over them.
+// Experts may also be plain, W_down act(W_up x) with act the square of relu (`act` 1).
 // Every sum runs over its row in one fixed order, so a token's result does not depend on what
 // else is in the batch.
 #include "common.h"
@@ -88,6 +95,132 @@ extern "C" int pylon_route_top(int* experts, float* weights, float* shared_gate,
   hipLaunchKernelGGL(route_top_kernel, dim3((tokens + 3) / 4), dim3(256), 0, stream, experts, weights, shared_gate,
                      logits, row_stride, bias, tokens, n_experts, top);
   PYLON_LAUNCHED("route_top");
+}
+
+#define MX_MAX_OUTPUTS (8 * PYLON_WAVE)
+
+__global__ void __launch_bounds__(256)
+route_scored_kernel(int* __restrict__ experts, float* __restrict__ weights, float* __restrict__ identity_weight,
+                    const float* __restrict__ logits, long long row_stride, const float* __restrict__ correction,
+                    int tokens, int n_outputs, int n_experts, int top, int groups, int keep, float scale) {
+  __shared__ float choice[4][MX_MAX_OUTPUTS];  // corrected scores, then -inf outside the kept groups
+  __shared__ float best_of[4][MX_MAX_OUTPUTS];  // every group's largest corrected score
+  const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= tokens) return;  // whole waves leave; only wave-level barriers follow
+  const float* row = logits + static_cast<size_t>(t) * row_stride;
+  float z[8], s[8];
+  float top_z = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int e = lane + PYLON_WAVE * i;
+    z[i] = e < n_outputs ? row[e] : -INFINITY;
+    top_z = fmaxf(top_z, z[i]);
+  }
+  top_z = wave_max(top_z);
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int e = lane + PYLON_WAVE * i;
+    s[i] = e < n_outputs ? expf(z[i] - top_z) : 0.f;
+    sum += s[i];
+  }
+  const float inv = 1.0f / wave_sum(sum);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int e = lane + PYLON_WAVE * i;
+    s[i] *= inv;
+    if (e < n_outputs) choice[wave][e] = s[i] + (correction != nullptr ? correction[e] : 0.f);
+  }
+  __builtin_amdgcn_wave_barrier();
+  const int per_group = n_outputs / groups;
+  if (keep < groups) {
+    for (int g = lane; g < groups; g += PYLON_WAVE) {
+      float m = -INFINITY;
+      for (int k = 0; k < per_group; ++k) m = fmaxf(m, choice[wave][g * per_group + k]);
+      best_of[wave][g] = m;
+    }
+    __builtin_amdgcn_wave_barrier();
+    // a group is kept if fewer than `keep` groups come before it (a larger score, or an equal one
+    // at a lower index)
+    for (int g = lane; g < groups; g += PYLON_WAVE) {
+      const float mine = best_of[wave][g];
+      int before = 0;
+      for (int o = 0; o < groups; ++o) {
+        const float other = best_of[wave][o];
+        before += (other > mine || (other == mine && o < g)) ? 1 : 0;
+      }
+      if (before >= keep)
+        for (int k = 0; k < per_group; ++k) choice[wave][g * per_group + k] = -INFINITY;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  float c[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int e = lane + PYLON_WAVE * i;
+    c[i] = e < n_outputs ? choice[wave][e] : -INFINITY;
+  }
+  float ident = 0.f;  // lane 0 adds up the identity experts' weights, in the order of the choices
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY, best_s = 0.f;
+    int best_e = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int e = lane + PYLON_WAVE * i;
+      if (e < n_outputs && c[i] != -INFINITY && (c[i] > best || (c[i] == best && e < best_e)) && !(c[i] != c[i])) {
+        best = c[i];
+        best_e = e;
+        best_s = s[i];
+      }
+    }
+#pragma unroll
+    for (int off = PYLON_WAVE / 2; off > 0; off >>= 1) {
+      const float other = __shfl_xor(best, off, PYLON_WAVE);
+      const int other_e = __shfl_xor(best_e, off, PYLON_WAVE);
+      const float other_s = __shfl_xor(best_s, off, PYLON_WAVE);
+      if (other_e != 0x7fffffff && (best_e == 0x7fffffff || other > best || (other == best && other_e < best_e))) {
+        best = other;
+        best_e = other_e;
+        best_s = other_s;
+      }
+    }
+    const bool none = best_e == 0x7fffffff;  // nothing comparable left: an identity of weight nothing
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (lane + PYLON_WAVE * i == best_e) c[i] = -INFINITY;
+    if (lane == 0) {
+      const float w = none ? 0.f : best_s * scale;
+      const bool identity = none || best_e >= n_experts;
+      experts[static_cast<size_t>(t) * top + k] = none ? n_outputs : best_e;
+      weights[static_cast<size_t>(t) * top + k] = identity ? 0.f : w;
+      if (identity) ident += w;
+    }
+  }
+  if (lane == 0 && identity_weight != nullptr) identity_weight[t] = ident;
+}
+
+// logits: float [tokens, n_outputs], rows row_stride apart; correction: null or float [n_outputs];
+// the first n_experts outputs are experts, the others identities.  experts int [tokens, top] (an
+// identity keeps its index, >= n_experts), weights float [tokens, top] (nothing for an identity),
+// identity_weight float [tokens] (null only if n_outputs == n_experts).
+extern "C" int pylon_route_scored(int* experts, float* weights, float* identity_weight, const float* logits,
+                                  long long row_stride, const float* correction, int tokens, int n_outputs,
+                                  int n_experts, int top, int groups, int keep, float scale, hipStream_t stream) {
+  PYLON_REQUIRE(tokens >= 0 && n_outputs >= 1 && n_outputs <= MX_MAX_OUTPUTS,
+                "route_scored: 1 to %d router outputs, got %d", MX_MAX_OUTPUTS, n_outputs);
+  PYLON_REQUIRE(n_experts >= 0 && n_experts <= n_outputs, "route_scored: %d experts among %d outputs", n_experts, n_outputs);
+  PYLON_REQUIRE(top >= 1 && top <= n_outputs && top <= MX_MAX_TOP, "route_scored: top %d of %d outputs (at most %d)",
+                top, n_outputs, MX_MAX_TOP);
+  PYLON_REQUIRE(groups >= 1 && n_outputs % groups == 0 && keep >= 1 && keep <= groups,
+                "route_scored: %d outputs do not form %d equal groups of which %d are kept", n_outputs, groups, keep);
+  PYLON_REQUIRE(row_stride >= n_outputs, "route_scored: rows of logits overlap");
+  PYLON_REQUIRE(identity_weight != nullptr || n_outputs == n_experts, "route_scored: identities need their weight's place");
+  if (tokens == 0) return 0;
+  hipLaunchKernelGGL(route_scored_kernel, dim3((tokens + 3) / 4), dim3(256), 0, stream, experts, weights,
+                     identity_weight, logits, row_stride, correction, tokens, n_outputs, n_experts, top, groups, keep,
+                     scale);
+  PYLON_LAUNCHED("route_scored");
 }
 
 // The dot product of a weight row with a vector in LDS, the lanes of a wave along the row: every
@@ -181,17 +314,46 @@ template <typename TX, typename TW>
 __global__ void __launch_bounds__(256)
 expert_gate_up_kernel(TX* __restrict__ hidden, const TX* __restrict__ x, long long x_stride,
                       const TW* __restrict__ w, long long w_stride, const int* __restrict__ experts, int top,
-                      int ff, int width, int units_per_block, int wide) {
+                      int ff, int width, int units_per_block, int wide, int act, int n_experts) {
   extern __shared__ float xs[];  // the token's input
   const int pair = blockIdx.y, t = pair / top;
   const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
+  const int e = experts[pair];
+  if (e >= n_experts) return;  // an identity: nothing to compute (the whole workgroup, before any barrier)
   for (int i = threadIdx.x; i < width; i += 256) xs[i] = to_float(x[static_cast<size_t>(t) * x_stride + i]);
   __syncthreads();
-  const int e = experts[pair];
-  const TW* gate = w + static_cast<size_t>(e) * 2 * ff * w_stride;
-  const TW* up = gate + static_cast<size_t>(ff) * w_stride;
   const int j0 = blockIdx.x * units_per_block;
   const int j1 = j0 + units_per_block < ff ? j0 + units_per_block : ff;
+  if (act == 1) {
+    // plain experts: hidden = relu(W_up x)^2, a wave four hidden units at a time
+    const TW* up1 = w + static_cast<size_t>(e) * ff * w_stride;
+    for (int j = j0 + 4 * wave; j < j1; j += 16) {
+      float share[4] = {0.f, 0.f, 0.f, 0.f};
+      bool done = false;
+      if constexpr (is_bf16<TW>::value) {
+        if (wide) {
+          const bf16_t* rows[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) rows[q] = up1 + static_cast<size_t>(j + q < j1 ? j + q : j1 - 1) * w_stride;
+          rows_dot_share<4, 2>(rows, xs, width, lane, share);
+          done = true;
+        }
+      }
+      if (!done) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (j + q < j1) share[q] = row_dot_share<TW>(up1 + static_cast<size_t>(j + q) * w_stride, xs, width, lane, wide);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float u = fmaxf(wave_sum(share[q]), 0.f);
+        if (lane == 0 && j + q < j1) hidden[static_cast<size_t>(pair) * ff + j + q] = from_float<TX>(u * u);
+      }
+    }
+    return;
+  }
+  const TW* gate = w + static_cast<size_t>(e) * 2 * ff * w_stride;
+  const TW* up = gate + static_cast<size_t>(ff) * w_stride;
   // a wave takes two hidden units at a time: the lanes' shares of all four rows first (their loads
   // are in flight together), then the four sums over the lanes
   for (int j = j0 + 2 * wave; j < j1; j += 8) {
@@ -225,9 +387,12 @@ expert_gate_up_kernel(TX* __restrict__ hidden, const TX* __restrict__ x, long lo
 
 // x: [tokens, width] (rows x_stride apart); w: [n_experts, 2 ff, width] (rows w_stride apart), an
 // expert's gate rows then its up rows; experts: int [tokens, top]; hidden: [tokens * top, ff].
+// act 1: plain experts, w [n_experts, ff, width], hidden = relu(W_up x)^2.  A pair whose expert is
+// n_experts or more (an identity) is passed over: its rows of hidden stay as they are.
 extern "C" int pylon_expert_gate_up(void* hidden, const void* x, int x_dtype, long long x_stride, const void* w,
                                     int w_dtype, long long w_stride, const int* experts, int tokens, int top, int ff,
-                                    int width, hipStream_t stream) {
+                                    int width, int act, int n_experts, hipStream_t stream) {
+  PYLON_REQUIRE(act == 0 || act == 1, "expert_gate_up: unknown activation %d", act);
   PYLON_REQUIRE(pylon_valid_dtype(x_dtype) && pylon_valid_dtype(w_dtype), "expert_gate_up: unknown dtype");
   PYLON_REQUIRE(!(x_dtype == PYLON_F32 && w_dtype == PYLON_BF16), "expert_gate_up: float inputs take float weights");
   PYLON_REQUIRE(tokens >= 0 && top >= 1 && ff >= 1 && width >= 1, "expert_gate_up: sizes must be positive");
@@ -249,7 +414,7 @@ extern "C" int pylon_expert_gate_up(void* hidden, const void* x, int x_dtype, lo
 #define GO(TX, TW)                                                                                               \
   hipLaunchKernelGGL((expert_gate_up_kernel<TX, TW>), grid, block, lds, stream, (TX*)hidden + off * ff,          \
                      (const TX*)x + (off / top) * x_stride, x_stride, (const TW*)w, w_stride, experts + off, top, \
-                     ff, width, units, wide)
+                     ff, width, units, wide, act, n_experts)
     if (x_dtype == PYLON_F32) GO(float, float);
     else if (w_dtype == PYLON_F32) GO(bf16_t, float);
     else GO(bf16_t, bf16_t);
@@ -263,12 +428,20 @@ __global__ void __launch_bounds__(256)
 expert_down_kernel(float* __restrict__ out, const TH* __restrict__ hidden, const TW* __restrict__ w,
                    long long w_stride, const int* __restrict__ experts, const float* __restrict__ weights,
                    const float* __restrict__ shared, const float* __restrict__ shared_gate, int top, int ff,
-                   int width, int cols_per_block, int wide) {
+                   int width, int cols_per_block, int wide, int n_experts, const TH* __restrict__ ident_x,
+                   long long ident_stride, const float* __restrict__ ident_w) {
   extern __shared__ float hs[];  // [top, ff]: the token's hidden activations of its chosen experts
   const int t = blockIdx.y;
   const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
-  for (int i = threadIdx.x; i < top * ff; i += 256) hs[i] = to_float(hidden[static_cast<size_t>(t) * top * ff + i]);
+  for (int i = threadIdx.x; i < top * ff; i += 256) {
+    // an identity's rows of hidden were never written
+    const bool real = experts[static_cast<size_t>(t) * top + i / ff] < n_experts;
+    hs[i] = real ? to_float(hidden[static_cast<size_t>(t) * top * ff + i]) : 0.f;
+  }
   __syncthreads();
+  // identity experts: the token's input itself, times the sum of their weights
+  const float iw = ident_w != nullptr ? ident_w[t] : 0.f;
+  const TH* ix = ident_x != nullptr ? ident_x + static_cast<size_t>(t) * ident_stride : nullptr;
   const int c0 = blockIdx.x * cols_per_block;
   const int c1 = c0 + cols_per_block < width ? c0 + cols_per_block : width;
   if constexpr (is_bf16<TW>::value) {
@@ -281,6 +454,7 @@ expert_down_kernel(float* __restrict__ out, const TH* __restrict__ hidden, const
       float share[4] = {0.f, 0.f, 0.f, 0.f};
       for (int s = 0; s < top; ++s) {
         const int e = experts[static_cast<size_t>(t) * top + s];
+        if (e >= n_experts) continue;
         const bf16_t* base = w + static_cast<size_t>(e) * width * w_stride;
         const bf16_t* rows[4];
 #pragma unroll
@@ -299,6 +473,7 @@ expert_down_kernel(float* __restrict__ out, const TH* __restrict__ hidden, const
             const float g = shared_gate != nullptr ? shared_gate[t] : 1.f;
             acc = fmaf(g, shared[static_cast<size_t>(t) * width + c + q], acc);
           }
+          if (ix != nullptr) acc = fmaf(iw, to_float(ix[c + q]), acc);
           out[static_cast<size_t>(t) * width + c + q] = acc;
         }
       }
@@ -311,6 +486,7 @@ expert_down_kernel(float* __restrict__ out, const TH* __restrict__ hidden, const
     float share = 0.f;
     for (int s = 0; s < top; ++s) {
       const int e = experts[static_cast<size_t>(t) * top + s];
+      if (e >= n_experts) continue;
       const TW* row = w + (static_cast<size_t>(e) * width + c) * w_stride;
       share = fmaf(weights[static_cast<size_t>(t) * top + s], row_dot_share<TW>(row, hs + s * ff, ff, lane, wide), share);
     }
@@ -320,6 +496,7 @@ expert_down_kernel(float* __restrict__ out, const TH* __restrict__ hidden, const
         const float g = shared_gate != nullptr ? shared_gate[t] : 1.f;
         acc = fmaf(g, shared[static_cast<size_t>(t) * width + c], acc);
       }
+      if (ix != nullptr) acc = fmaf(iw, to_float(ix[c]), acc);
       out[static_cast<size_t>(t) * width + c] = acc;
     }
   }
@@ -327,11 +504,15 @@ expert_down_kernel(float* __restrict__ out, const TH* __restrict__ hidden, const
 
 // hidden: [tokens * top, ff]; w: [n_experts, width, ff] (rows w_stride apart); experts int and
 // weights float [tokens, top]; shared: null or float [tokens, width], multiplied by shared_gate[t]
-// (null: by one) and added; out: float [tokens, width].
+// (null: by one) and added; out: float [tokens, width].  A pair whose expert is n_experts or more is
+// passed over; ident_x (null, or [tokens, width] of h_dtype, rows ident_stride apart) times
+// ident_w[t] is added: the identity experts' share.
 extern "C" int pylon_expert_down(float* out, const void* hidden, int h_dtype, const void* w, int w_dtype,
                                  long long w_stride, const int* experts, const float* weights, const float* shared,
-                                 const float* shared_gate, int tokens, int top, int ff, int width,
+                                 const float* shared_gate, int tokens, int top, int ff, int width, int n_experts,
+                                 const void* ident_x, long long ident_stride, const float* ident_w,
                                  hipStream_t stream) {
+  PYLON_REQUIRE((ident_x == nullptr) == (ident_w == nullptr), "expert_down: identities need inputs and weights");
   PYLON_REQUIRE(pylon_valid_dtype(h_dtype) && pylon_valid_dtype(w_dtype), "expert_down: unknown dtype");
   PYLON_REQUIRE(!(h_dtype == PYLON_F32 && w_dtype == PYLON_BF16), "expert_down: float inputs take float weights");
   PYLON_REQUIRE(tokens >= 0 && top >= 1 && ff >= 1 && width >= 1, "expert_down: sizes must be positive");
@@ -350,7 +531,9 @@ extern "C" int pylon_expert_down(float* out, const void* hidden, int h_dtype, co
   hipLaunchKernelGGL((expert_down_kernel<TH, TW>), grid, block, lds, stream, out + off * width,                 \
                      (const TH*)hidden + off * top * ff, (const TW*)w, w_stride, experts + off * top,           \
                      weights + off * top, shared != nullptr ? shared + off * width : nullptr,                   \
-                     shared_gate != nullptr ? shared_gate + off : nullptr, top, ff, width, cols, wide)
+                     shared_gate != nullptr ? shared_gate + off : nullptr, top, ff, width, cols, wide, n_experts, \
+                     ident_x != nullptr ? (const TH*)ident_x + off * ident_stride : nullptr, ident_stride,      \
+                     ident_w != nullptr ? ident_w + off : nullptr)
     if (h_dtype == PYLON_F32) GO(float, float);
     else if (w_dtype == PYLON_F32) GO(bf16_t, float);
     else GO(bf16_t, bf16_t);
@@ -374,11 +557,12 @@ typedef float mx_floatx4 __attribute__((ext_vector_type(4)));
 
 #define MX_WAVE_COLS 32
 
-template <bool GLU, int MT, typename TO>
+template <int ACT, int MT, typename TO>
 __global__ void __launch_bounds__(256)
 grouped_rows_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restrict__ x, long long ldx,
                     const int* __restrict__ row_index, const uint16_t* __restrict__ w, long long ldw,
                     long long expert_rows, const int* __restrict__ offsets, int n_experts, int N, int K) {
+  constexpr bool GLU = ACT == 1;  // ACT: 0 the sums as they are, 1 silu(gate) * up, 2 the square of relu
   constexpr int MX_TM = 16 * MT;  // rows of a tile
   constexpr int J = GLU ? 4 : 2;  // weight tiles of a wave: GLU: two of gate rows, then the two of their up rows
   const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
@@ -457,6 +641,7 @@ grouped_rows_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restr
         if (n >= N) continue;
         float v = acc[j][t][i];
         if constexpr (GLU) v = v / (1.0f + expf(-v)) * acc[2 + j][t][i];
+        if constexpr (ACT == 2) v = fmaxf(v, 0.f) * fmaxf(v, 0.f);
         orow[n] = from_float<TO>(v);
       }
   }
@@ -474,11 +659,12 @@ grouped_rows_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restr
 #define GT_K 64
 #define GT_PITCH 144
 
-template <bool GLU, typename TO>
+template <int ACT, typename TO>
 __global__ void __launch_bounds__(256, 2)
 grouped_tiles_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restrict__ x, long long ldx,
                      const int* __restrict__ row_index, const uint16_t* __restrict__ w, long long ldw,
                      long long expert_rows, const int* __restrict__ offsets, int n_experts, int N, int K) {
+  constexpr bool GLU = ACT == 1;
   constexpr int WROWS = 2 * GT_COLS;  // GLU: 128 gate rows and their 128 up rows; else 256 output columns
   constexpr int TILE_COLS = GLU ? GT_COLS : 2 * GT_COLS, WAVE_COLS = TILE_COLS / 4;
   constexpr int XLOADS = GT_ROWS / 32, LOADS = (GT_ROWS + WROWS) / 32;
@@ -569,6 +755,7 @@ grouped_tiles_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __rest
         if (n >= N) continue;
         float v = acc[j][t][i];
         if constexpr (GLU) v = v / (1.0f + expf(-v)) * acc[2 + j][t][i];
+        if constexpr (ACT == 2) v = fmaxf(v, 0.f) * fmaxf(v, 0.f);
         orow[n] = from_float<TO>(v);
       }
   }
@@ -593,22 +780,41 @@ static int grouped_checks(const char* name, const void* x, long long ldx, const 
 
 // hidden[p] = silu(W_gate[e] x[row_index[p]]) * (W_up[e] x[row_index[p]]) for the sorted pairs p of
 // every expert e (offsets: int [n_experts + 1]); x bfloat16 [tokens, width]; w bfloat16
-// [n_experts * 2 ff, width]; hidden bfloat16 [pairs, ff]; tokens_bound: the rows of x.
+// [n_experts * 2 ff, width]; hidden bfloat16 [pairs, ff]; tokens_bound: the rows of x.  act 1: plain
+// experts, hidden[p] = relu(W_up[e] x)^2 with w [n_experts * ff, width].  pairs counts the sorted
+// pairs of these n_experts experts only (identities' pairs lie behind them).
 extern "C" int pylon_grouped_gate_up(void* hidden, const void* x, long long ldx, const int* row_index, const void* w,
                                      long long ldw, const int* offsets, int pairs, int n_experts, int ff, int width,
-                                     int tokens_bound, hipStream_t stream) {
+                                     int tokens_bound, int act, hipStream_t stream) {
   if (grouped_checks("grouped_gate_up", x, ldx, w, ldw, width, ff, pairs, n_experts)) return 1;
+  PYLON_REQUIRE(act == 0 || act == 1, "grouped_gate_up: unknown activation %d", act);
   if (pairs == 0) return 0;
+  if (act == 1) {
+    // plain experts: w [n_experts * ff, width], hidden = relu(W_up x)^2; tiles of 256 columns where large
+    const bool large1 = grouped_large(pairs, n_experts, tokens_bound * ldx, 1ll * n_experts * ff * ldw);
+    const int tile1 = large1 ? GT_ROWS : 64, cols1 = large1 ? 2 * GT_COLS : 4 * MX_WAVE_COLS;
+    dim3 grid1(pairs / tile1 + n_experts, (ff + cols1 - 1) / cols1), block1(256);
+    PYLON_REQUIRE(grid1.y <= 65535, "grouped_gate_up: too many columns for one launch");
+    if (large1)
+      hipLaunchKernelGGL((grouped_tiles_kernel<2, bf16_t>), grid1, block1, 0, stream, (bf16_t*)hidden, (long long)ff,
+                         (const uint16_t*)x, ldx, row_index, (const uint16_t*)w, ldw, (long long)ff, offsets, n_experts,
+                         ff, width);
+    else
+      hipLaunchKernelGGL((grouped_rows_kernel<2, 4, bf16_t>), grid1, block1, 0, stream, (bf16_t*)hidden, (long long)ff,
+                         (const uint16_t*)x, ldx, row_index, (const uint16_t*)w, ldw, (long long)ff, offsets, n_experts,
+                         ff, width);
+    PYLON_LAUNCHED("grouped_gate_up");
+  }
   const bool large = grouped_large(pairs, n_experts, tokens_bound * ldx, 2ll * n_experts * ff * ldw);
   const int tile = large ? GT_ROWS : 64;
   dim3 grid(pairs / tile + n_experts, (ff + 4 * MX_WAVE_COLS - 1) / (4 * MX_WAVE_COLS)), block(256);
   PYLON_REQUIRE(grid.y <= 65535, "grouped_gate_up: too many columns for one launch");
   if (large)
-    hipLaunchKernelGGL((grouped_tiles_kernel<true, bf16_t>), grid, block, 0, stream, (bf16_t*)hidden, (long long)ff,
+    hipLaunchKernelGGL((grouped_tiles_kernel<1, bf16_t>), grid, block, 0, stream, (bf16_t*)hidden, (long long)ff,
                        (const uint16_t*)x, ldx, row_index, (const uint16_t*)w, ldw, 2ll * ff, offsets, n_experts, ff,
                        width);
   else
-    hipLaunchKernelGGL((grouped_rows_kernel<true, 4, bf16_t>), grid, block, 0, stream, (bf16_t*)hidden,
+    hipLaunchKernelGGL((grouped_rows_kernel<1, 4, bf16_t>), grid, block, 0, stream, (bf16_t*)hidden,
                        (long long)ff, (const uint16_t*)x, ldx, row_index, (const uint16_t*)w, ldw, 2ll * ff, offsets,
                        n_experts, ff, width);
   PYLON_LAUNCHED("grouped_gate_up");
@@ -626,11 +832,11 @@ extern "C" int pylon_grouped_down(float* y, const void* hidden, long long ldh, c
   dim3 grid(pairs / tile + n_experts, (width + cols - 1) / cols), block(256);
   PYLON_REQUIRE(grid.y <= 65535, "grouped_down: too many columns for one launch");
   if (large)
-    hipLaunchKernelGGL((grouped_tiles_kernel<false, float>), grid, block, 0, stream, y, (long long)width,
+    hipLaunchKernelGGL((grouped_tiles_kernel<0, float>), grid, block, 0, stream, y, (long long)width,
                        (const uint16_t*)hidden, ldh, nullptr, (const uint16_t*)w, ldw, (long long)width, offsets,
                        n_experts, width, ff);
   else
-    hipLaunchKernelGGL((grouped_rows_kernel<false, 4, float>), grid, block, 0, stream, y, (long long)width,
+    hipLaunchKernelGGL((grouped_rows_kernel<0, 4, float>), grid, block, 0, stream, y, (long long)width,
                        (const uint16_t*)hidden, ldh, nullptr, (const uint16_t*)w, ldw, (long long)width, offsets,
                        n_experts, width, ff);
   PYLON_LAUNCHED("grouped_down");
@@ -639,30 +845,43 @@ extern "C" int pylon_grouped_down(float* y, const void* hidden, long long ldh, c
 __global__ void __launch_bounds__(256)
 expert_combine_kernel(float* __restrict__ out, const float* __restrict__ y, const int* __restrict__ place,
                       const float* __restrict__ weights, const float* __restrict__ shared,
-                      const float* __restrict__ shared_gate, int top, int width) {
+                      const float* __restrict__ shared_gate, int top, int width, const int* __restrict__ real_end,
+                      const uint16_t* __restrict__ ident_x, long long ident_stride, const float* __restrict__ ident_w) {
   const int t = blockIdx.y;
   const int c = blockIdx.x * 256 + threadIdx.x;
   if (c >= width) return;
   float acc = 0.f;
-  for (int s = 0; s < top; ++s)
-    acc = fmaf(weights[static_cast<size_t>(t) * top + s], y[static_cast<size_t>(place[static_cast<size_t>(t) * top + s]) * width + c], acc);
+  const int real_pairs = real_end != nullptr ? real_end[0] : 0x7fffffff;
+  for (int s = 0; s < top; ++s) {
+    const int p = place[static_cast<size_t>(t) * top + s];
+    if (p >= real_pairs) continue;  // an identity's pair: no expert has written its row of y
+    acc = fmaf(weights[static_cast<size_t>(t) * top + s], y[static_cast<size_t>(p) * width + c], acc);
+  }
   if (shared != nullptr) acc = fmaf(shared_gate != nullptr ? shared_gate[t] : 1.f, shared[static_cast<size_t>(t) * width + c], acc);
+  if (ident_x != nullptr)
+    acc = fmaf(ident_w[t], bf16_bits_to_float(ident_x[static_cast<size_t>(t) * ident_stride + c]), acc);
   out[static_cast<size_t>(t) * width + c] = acc;
 }
 
 // out[t] = sum_s weights[t, s] y[place[t, s]] (+ shared_gate[t] * shared[t]): the experts' outputs of
 // the sorted pairs brought back to their tokens, in the order of the token's choices.
+// Sorted pairs from real_end[0] on (null: none) belong to identity experts: ident_x (null, or bfloat16 [tokens, width],
+// rows ident_stride apart) times ident_w[t] stands for them.
 extern "C" int pylon_expert_combine(float* out, const float* y, const int* place, const float* weights,
                                     const float* shared, const float* shared_gate, int tokens, int top, int width,
+                                    const int* real_end, const void* ident_x, long long ident_stride, const float* ident_w,
                                     hipStream_t stream) {
   PYLON_REQUIRE(tokens >= 0 && top >= 1 && width >= 1, "expert_combine: sizes must be positive");
+  PYLON_REQUIRE((ident_x == nullptr) == (ident_w == nullptr), "expert_combine: identities need inputs and weights");
   if (tokens == 0) return 0;
   for (int first = 0; first < tokens; first += 65535) {
     const int n = tokens - first < 65535 ? tokens - first : 65535;
     const size_t off = static_cast<size_t>(first);
     hipLaunchKernelGGL(expert_combine_kernel, dim3((width + 255) / 256, n), dim3(256), 0, stream, out + off * width, y,
                        place + off * top, weights + off * top, shared != nullptr ? shared + off * width : nullptr,
-                       shared_gate != nullptr ? shared_gate + off : nullptr, top, width);
+                       shared_gate != nullptr ? shared_gate + off : nullptr, top, width, real_end,
+                       ident_x != nullptr ? (const uint16_t*)ident_x + off * ident_stride : nullptr, ident_stride,
+                       ident_w != nullptr ? ident_w + off : nullptr);
   }
   PYLON_LAUNCHED("expert_combine");
 }

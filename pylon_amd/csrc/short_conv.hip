@@ -119,3 +119,59 @@ extern "C" int pylon_short_conv(void* out, int out_dtype, const void* h, int in_
 #undef GO
   PYLON_LAUNCHED("short_conv");
 }
+
+// ---- token shift -------------------------------------------------------------------------------
+//   out[t, c] = h[t, c] + (h[t - 1, c] - h[t, c]) * shift[c]
+// with zeros before a request's first token; a request's last input is kept in its state slot,
+// float [width].  Tiles and the ownership of the state as in the convolution above: the thread with
+// a row's first tile reads the old state, and writes the new one after it has read the old.
+template <typename TI, typename TO>
+__global__ void token_shift_kernel(TO* __restrict__ out, const TI* __restrict__ h, const float* __restrict__ shift,
+                                   float* state, const int* __restrict__ row_start,
+                                   const int* __restrict__ row_slots, int tiles_per_row, int width) {
+  const int row = blockIdx.x / tiles_per_row;
+  const int tile = blockIdx.x - row * tiles_per_row;
+  const int begin = row_start[row], end = row_start[row + 1];
+  const int a = begin + tile * CONV_TILE;
+  if (a >= end) return;
+  const int b = a + CONV_TILE < end ? a + CONV_TILE : end;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  float* st = state + static_cast<size_t>(row_slots[row]) * width + c;
+  const float s = shift[c];
+  float prev = tile == 0 ? st[0] : to_float(h[static_cast<size_t>(a - 1) * width + c]);
+  float xs[CONV_TILE];
+#pragma unroll
+  for (int n = 0; n < CONV_TILE; ++n) xs[n] = (a + n < b) ? to_float(h[static_cast<size_t>(a + n) * width + c]) : 0.f;
+#pragma unroll
+  for (int n = 0; n < CONV_TILE; ++n) {
+    if (a + n >= b) break;
+    const float x = xs[n];
+    out[static_cast<size_t>(a + n) * width + c] = from_float<TO>(fmaf(prev - x, s, x));
+    prev = x;
+  }
+  if (tile == 0) st[0] = to_float(h[static_cast<size_t>(end - 1) * width + c]);
+}
+
+// h: [tokens, width] of in_dtype; shift: float [width]; out: [tokens, width] of out_dtype; state: float
+// [slots, width]; row_start, row_slots, max_count as for the convolution.
+extern "C" int pylon_token_shift(void* out, int out_dtype, const void* h, int in_dtype, const float* shift,
+                                 float* state, const int* row_start, const int* row_slots, int rows, int max_count,
+                                 int width, hipStream_t stream) {
+  PYLON_REQUIRE(pylon_valid_dtype(out_dtype) && pylon_valid_dtype(in_dtype), "token_shift: unknown dtype");
+  PYLON_REQUIRE(rows >= 0 && max_count >= 0 && width > 0, "token_shift: bad sizes");
+  PYLON_REQUIRE(state != nullptr && shift != nullptr, "token_shift: the state and the weights are required");
+  if (rows == 0 || max_count == 0) return 0;
+  const int tiles_per_row = (max_count + CONV_TILE - 1) / CONV_TILE;
+  PYLON_REQUIRE(static_cast<long long>(rows) * tiles_per_row < (1ll << 31), "token_shift: too many tiles");
+  dim3 grid(static_cast<unsigned>(rows * tiles_per_row), (width + 255) / 256), block(256);
+#define GO(TI, TO)                                                                                        \
+  hipLaunchKernelGGL((token_shift_kernel<TI, TO>), grid, block, 0, stream, (TO*)out, (const TI*)h, shift, \
+                     state, row_start, row_slots, tiles_per_row, width)
+  if (in_dtype == PYLON_F32 && out_dtype == PYLON_F32) GO(float, float);
+  else if (in_dtype == PYLON_F32) GO(float, bf16_t);
+  else if (out_dtype == PYLON_F32) GO(bf16_t, float);
+  else GO(bf16_t, bf16_t);
+#undef GO
+  PYLON_LAUNCHED("token_shift");
+}

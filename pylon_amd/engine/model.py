@@ -13,6 +13,7 @@ before its run: how a model that runs a stretch of layers several times feeds ev
 """
 from __future__ import annotations
 
+from dataclasses import replace
 from typing import List, Optional
 
 import torch
@@ -20,7 +21,7 @@ import torch
 from ..config.specs import ModelSpec
 from ..kernels import ops
 from ..parts import build_part
-from ..parts.base import Part
+from ..parts.base import KVRequirement, Part, requirement_list
 from .batch import StepContext
 
 
@@ -52,17 +53,26 @@ class Model(Part):
 
     # ---- what the cache manager has to provide ------------------------------------------
     def cache_requirements(self) -> List[object]:
-        """Per run of the schedule: what its mixer keeps (None for a run that borrows)."""
+        """Per run of the schedule: what it keeps.  A run that borrows another run's keys and values
+        keeps none of its own, but its fixed-size state (a token shift's last input, a convolution's
+        window) is its own."""
+        def split(need):
+            parts = requirement_list(need)
+            return ([p for p in parts if isinstance(p, KVRequirement)],
+                    [p for p in parts if not isinstance(p, KVRequirement)])
+
         needs: List[object] = []
-        for layer, cache_id, stores in self.schedule:
-            needs.append(self.blocks[layer].cache_requirement() if stores else None)
         for index, (layer, cache_id, stores) in enumerate(self.schedule):
-            if not stores:
-                own = self.blocks[layer].cache_requirement()
-                if own != needs[cache_id]:
-                    raise ValueError(
-                        f"run {index} borrows the cache of run {cache_id}, which has another geometry"
-                    )
+            own = self.blocks[layer].cache_requirement()
+            if stores:
+                needs.append(own)
+                continue
+            kv, states = split(own)
+            if kv != split(self.blocks[self.schedule[cache_id][0]].cache_requirement())[0]:
+                raise ValueError(
+                    f"run {index} borrows the cache of run {cache_id}, which has another geometry"
+                )
+            needs.append(None if not states else (states[0] if len(states) == 1 else tuple(states)))
         return needs
 
     def decode_signature(self, rows: int, bound: int) -> tuple:
@@ -93,10 +103,15 @@ class Model(Part):
         # a schedule may add the embedded tokens to the stream again before some of its runs
         embedded = resid.clone() if any(self.embedding_again) else None
         delta = None
-        for (layer, cache_id, stores), again in zip(self.schedule, self.embedding_again):
+        for run, ((layer, cache_id, stores), again) in enumerate(zip(self.schedule, self.embedding_again)):
             if again:
                 ops.residual_add(resid, embedded)  # the pending output of the run before follows in the norm
-            resid, delta = self.blocks[layer].forward(resid, delta, ctx, ctx.cache(cache_id), stores)
+            cache = ctx.cache(cache_id)
+            if not stores:
+                # the lender's keys and values, the run's own fixed-size state
+                own = ctx.cache(run)
+                cache = replace(cache, state=own.state, states=own.states)
+            resid, delta = self.blocks[layer].forward(resid, delta, ctx, cache, stores)
         if ctx.n_logits == 0:
             return None
         h = self.final_norm.add_forward(resid, delta, row_idx=ctx.logit_idx)

@@ -212,14 +212,16 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     page_size: int, window: Optional[int], scale: float,
                     out: Optional[torch.Tensor] = None, rel: Optional[torch.Tensor] = None,
                     bucket: Optional[torch.Tensor] = None, sink: bool = False,
-                    v_transposed: bool = False, chunk: Optional[int] = None) -> torch.Tensor:
+                    v_transposed: bool = False, chunk: Optional[int] = None,
+                    log_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention of each token over its request's cached keys ``<=`` its position (with
     ``window`` the last so many, with ``chunk`` those of its own chunk: :func:`mask_code`).
     ``q`` is ``[tokens, heads, head_dim]`` and may be a slice of wider rows (a fused
     projection); values may have another size than keys.  ``rel`` (float32 ``[rows, heads]``)
     with ``bucket`` (int32 ``[n]``) adds ``rel[bucket[min(i - j, n - 1)], head]`` to the scaled
-    score of query ``i`` and key ``j``; ``sink`` adds one to the softmax's denominator.  With
-    ``v_transposed`` the values lie as ``[pages, kv_heads, v_dim, page_size]``."""
+    score of query ``i`` and key ``j``; ``log_bias`` (float32 ``[2, heads]``: ``a`` then ``b``) takes
+    ``a[head] * log(1 + b[head] * (i - j))`` off it instead; ``sink`` adds one to the softmax's
+    denominator.  With ``v_transposed`` the values lie as ``[pages, kv_heads, v_dim, page_size]``."""
     if q.dim() != 3:
         raise KernelError("paged_attention takes q as [tokens, heads, head_dim]")
     tokens, n_heads, head_dim = q.shape
@@ -237,6 +239,10 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         raise KernelError("paged_attention: rel and bucket go together")
     if rel is not None and (rel.dim() != 2 or rel.shape[1] != n_heads or bucket.numel() < 1):
         raise KernelError("paged_attention: rel must be [rows, heads] and bucket hold at least one entry")
+    if log_bias is not None:
+        if rel is not None or log_bias.shape != (2, n_heads) or not log_bias.is_contiguous():
+            raise KernelError("paged_attention: log_bias is float32 [2, heads], and not together with a table")
+        rel = log_bias
     if psize != page_size or hd != head_dim:
         raise KernelError("paged_attention: cache geometry does not match page_size/head_dim")
     if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
@@ -267,11 +273,10 @@ SINK_MAX_BIAS = 4096  # distances the matrix-core sink attention keeps a bias fo
 SINK_TILE = 32        # most tokens of one tile of it
 
 
-def attention_sink_ok(dtype: torch.dtype, *, head_dim: int, v_dim: int, page_size: int, bucket_len: int,
-                      window: Optional[int] = None) -> bool:
+def attention_sink_ok(dtype: torch.dtype, *, head_dim: int, v_dim: int, page_size: int, bucket_len: int) -> bool:
     """Whether the matrix-core kernel takes this geometry (else the general kernel does)."""
     return (dtype == torch.bfloat16 and head_dim % 8 == 0 and 8 <= head_dim <= 256 and v_dim % 4 == 0
-            and 4 <= v_dim <= 256 and page_size % 32 == 0 and bucket_len <= SINK_MAX_BIAS and window is None)
+            and 4 <= v_dim <= 256 and page_size % 32 == 0 and bucket_len <= SINK_MAX_BIAS)
 
 
 def sink_cuts(tokens: int, n_heads: int, n_kv_heads: int, max_len: int, units: Optional[int] = None) -> int:
@@ -295,14 +300,16 @@ def bias_by_distance(rel: torch.Tensor, bucket: torch.Tensor) -> torch.Tensor:
 
 def attention_sink(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                    tiles: Optional[torch.Tensor], positions: Optional[torch.Tensor], *, page_size: int, scale: float,
-                   bias: Optional[torch.Tensor], sink: bool, cuts: int = 1) -> torch.Tensor:
+                   bias: Optional[torch.Tensor], sink: bool, cuts: int = 1, window: Optional[int] = None,
+                   chunk: Optional[int] = None) -> torch.Tensor:
     """Causal attention with a bias by distance and a sink on the matrix cores: bfloat16 ``q``
     ``[tokens, heads, head_dim]`` (maybe a slice of wider rows), keys ``[pages, page_size, kv_heads,
     head_dim]``, values transposed inside their pages ``[pages, kv_heads, v_dim, page_size]``.
     ``bias`` float32 ``[heads, n]``: what is added to the scaled score at distance ``min(i - j, n - 1)``.
     ``tiles`` int32 ``[n, 4]`` (first token, count <= 32, block-table row, first position); or None
     with ``positions``: every token a tile of its own on its own row of the table.  ``cuts``
-    workgroups share the keys of a tile and a second kernel merges their float partial results."""
+    workgroups share the keys of a tile and a second kernel merges their float partial results.
+    ``window`` / ``chunk``: which earlier keys a token sees (:func:`mask_code`)."""
     if q.dim() != 3 or k_cache.dim() != 4 or v_cache.dim() != 4:
         raise KernelError("attention_sink takes q [tokens, heads, head_dim] and 4-D caches")
     tokens, n_heads, head_dim = q.shape
@@ -337,22 +344,30 @@ def attention_sink(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
               _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32),
               block_table.shape[1], _dev(tiles, "tiles", torch.int32), _dev(positions, "positions", torch.int32),
               n_tiles, n_heads, n_kv_heads, head_dim, v_dim, page_size, float(scale), _dev(bias, "bias", torch.float32),
-              0 if bias is None else bias.shape[1], 1 if sink else 0, int(cuts), _dev(partial, "partial"), 0 if partial is None else partial.numel(), tokens, _stream())
+              0 if bias is None else bias.shape[1], 1 if sink else 0, int(cuts), _dev(partial, "partial"),
+              0 if partial is None else partial.numel(), tokens, mask_code(window, chunk), _stream())
     return out
 
 
 def add_normed_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], gain: Optional[torch.Tensor], eps: float,
                        out_dtype: Optional[torch.dtype], *, post_gain: Optional[torch.Tensor] = None,
-                       post_eps: float = 0.0, row_idx: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+                       post_eps: float = 0.0, row_idx: Optional[torch.Tensor] = None,
+                       delta_scale: Optional[torch.Tensor] = None,
+                       delta_bias: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """``resid += post_gain * d / rms(d)`` (``d`` = ``delta``, or the sum of a stack of float32
     partial sums; without ``post_gain``: ``resid += d``), in float32 and in place, then
     ``gain * resid / rms(resid)`` in ``out_dtype``, with ``rms(v) = sqrt(mean(v^2) + eps)``.
     ``post_gain`` is one float32 number on the device; ``gain`` one number or one per element.
     With ``row_idx`` only those rows are normed and ``resid`` is left as it is; with
-    ``gain`` None only the sum is formed."""
+    ``gain`` None only the sum is formed.  ``delta_bias`` (float32 ``[dim]``) is added to ``d``
+    first; with ``delta_scale`` (float32 ``[dim]``, not together with ``post_gain``) the sum is
+    ``resid += delta_scale * d``."""
     if resid.dim() != 2:
         raise KernelError("add_normed_rmsnorm takes a 2-D residual")
     dim = resid.shape[1]
+    for name, vector in (("delta_scale", delta_scale), ("delta_bias", delta_bias)):
+        if vector is not None and (vector.shape != (dim,) or delta is None):
+            raise KernelError(f"add_normed_rmsnorm: {name} is one number per element of an output that is given")
     n_delta, delta_stride = 1, 0
     if delta is not None:
         if delta.dim() == 3:
@@ -377,8 +392,89 @@ def add_normed_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], gain:
               _dev(resid, "resid", torch.float32), _dev(delta, "delta"),
               dtype_code(delta.dtype) if delta is not None else F32, n_delta, delta_stride,
               _dev(post_gain, "post_gain", torch.float32), float(post_eps), _dev(gain, "gain", torch.float32),
-              gain_stride, _dev(row_idx, "row_idx", torch.int32), rows, dim, float(eps), _stream())
+              gain_stride, _dev(row_idx, "row_idx", torch.int32), rows, dim, float(eps),
+              _dev(delta_scale, "delta_scale", torch.float32), _dev(delta_bias, "delta_bias", torch.float32), _stream())
     return out
+
+
+def depth_mix(resid: torch.Tensor, delta: Optional[torch.Tensor], streams: torch.Tensor, index: int,
+              coeff: torch.Tensor, *, delta_scale: Optional[torch.Tensor] = None,
+              delta_bias: Optional[torch.Tensor] = None, gain: Optional[torch.Tensor] = None, eps: float = 0.0,
+              out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """A layer's result joins the earlier layers' and the stream becomes their learned mix:
+    ``X = resid + delta_scale * (d + delta_bias)`` (``d`` = ``delta`` or the sum of a stack of partial
+    sums; scale and bias optional), ``streams[index] = X``, ``resid = sum_{j <= index} coeff[j] *
+    streams[j]``, all float32 and in place; with ``gain`` (float32 ``[dim]``) also the norm
+    ``gain * resid / sqrt(mean(resid^2) + eps)`` in ``out_dtype``.  ``streams`` is float32
+    ``[n, tokens, dim]`` with ``n > index``; ``coeff`` float32 with at least ``index + 1`` numbers."""
+    if resid.dim() != 2 or resid.dtype != torch.float32 or not resid.is_contiguous():
+        raise KernelError("depth_mix takes a contiguous float32 2-D residual")
+    rows, dim = resid.shape
+    if (streams.dim() != 3 or streams.dtype != torch.float32 or streams.shape[1:] != resid.shape
+            or not streams.is_contiguous() or not 0 <= index < streams.shape[0]):
+        raise KernelError("depth_mix: streams must be float32 [more than index, tokens, dim]")
+    if coeff.dim() != 1 or coeff.numel() < index + 1:
+        raise KernelError(f"depth_mix: stream {index} needs {index + 1} coefficients")
+    n_delta, delta_stride = 1, 0
+    if delta is not None:
+        if delta.dim() == 3:
+            n_delta, delta_stride = delta.shape[0], delta.shape[1] * delta.shape[2]
+            if delta.shape[1:] != resid.shape:
+                raise KernelError("depth_mix: partial sums and resid differ in shape")
+        elif delta.shape != resid.shape:
+            raise KernelError("depth_mix: delta and resid differ in shape")
+    for name, vector in (("delta_scale", delta_scale), ("delta_bias", delta_bias), ("gain", gain)):
+        if vector is not None and vector.shape != (dim,):
+            raise KernelError(f"depth_mix: {name} is one number per element")
+    out = None if gain is None else torch.empty((rows, dim), dtype=out_dtype, device=resid.device)
+    _lib.call("pylon_depth_mix", _dev(out, "out"), dtype_code(out.dtype) if out is not None else F32,
+              _dev(resid, "resid", torch.float32), _dev(delta, "delta"),
+              dtype_code(delta.dtype) if delta is not None else F32, n_delta, delta_stride,
+              _dev(delta_scale, "delta_scale", torch.float32), _dev(delta_bias, "delta_bias", torch.float32),
+              _dev(streams, "streams", torch.float32), rows * dim, int(index), _dev(coeff, "coeff", torch.float32),
+              _dev(gain, "gain", torch.float32), rows, dim, float(eps), _stream())
+    return out
+
+
+def token_shift(h: torch.Tensor, shift: torch.Tensor, state: torch.Tensor, row_start: torch.Tensor,
+                row_slots: torch.Tensor, *, rows: int, max_count: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """``h[t] + (h[t - 1] - h[t]) * shift`` per channel and request, zeros before a request's first
+    token.  ``state`` (float32 ``[slots, width]``) holds every request's last input and is brought
+    up to date; ``max_count`` bounds the tokens of a row."""
+    if h.dim() != 2 or shift.shape != (h.shape[1],) or not h.is_contiguous():
+        raise KernelError("token_shift takes h [tokens, width] and one weight per channel")
+    tokens, width = h.shape
+    if state is None or state.dim() != 2 or state.shape[1] != width:
+        raise KernelError(f"token_shift: state must be [slots, {width}]")
+    if row_start.numel() != rows + 1 or row_slots.numel() != rows:
+        raise KernelError("token_shift: one start per row and one more, and one slot per row")
+    out = torch.empty((tokens, width), dtype=out_dtype, device=h.device)
+    _lib.call("pylon_token_shift", _dev(out, "out"), dtype_code(out_dtype), _dev(h, "h"), dtype_code(h.dtype),
+              _dev(shift, "shift", torch.float32), _dev(state, "state", torch.float32),
+              _dev(row_start, "row_start", torch.int32), _dev(row_slots, "row_slots", torch.int32), rows,
+              int(max_count), width, _stream())
+    return out
+
+
+def add_sinusoid(x: torch.Tensor, positions: torch.Tensor, freq: torch.Tensor) -> torch.Tensor:
+    """``x[t, 2i] += sin(p_t * freq[i])``, ``x[t, 2i + 1] += cos(p_t * freq[i])`` in place (float32)."""
+    if x.dim() != 2 or x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelError("add_sinusoid takes a contiguous float32 [tokens, dim]")
+    tokens, dim = x.shape
+    if positions.numel() != tokens or freq.numel() != (dim + 1) // 2:
+        raise KernelError("add_sinusoid: one position per token and one frequency per pair of elements")
+    _lib.call("pylon_add_sinusoid", _dev(x, "x", torch.float32), _dev(positions, "positions", torch.int32),
+              _dev(freq, "freq", torch.float32), tokens, dim, _stream())
+    return x
+
+
+def add_bias_(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """``x[..., i] += bias[i]`` in place; ``x`` contiguous, ``bias`` float32 of the last axis' length."""
+    if not x.is_contiguous() or bias.shape != (x.shape[-1],):
+        raise KernelError("add_bias_ takes a contiguous tensor and one bias per element of its last axis")
+    _lib.call("pylon_add_bias", _dev(x, "x"), dtype_code(x.dtype), _dev(bias, "bias", torch.float32),
+              x.numel() // x.shape[-1], x.shape[-1], _stream())
+    return x
 
 
 def short_conv(h: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tensor], row_start: torch.Tensor,
@@ -499,17 +595,52 @@ def kv_store(proj: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, s
               tokens, k_row, v_row, page_size if v_transposed else 0, _stream())
 
 
+def qkv_bias_store(proj: torch.Tensor, bias: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                   v_cache: Optional[torch.Tensor], slot_map: Optional[torch.Tensor], *, q_size: int, k_size: int,
+                   v_size: int, out_dtype: torch.dtype, store: bool, v_transposed: bool = False) -> torch.Tensor:
+    """A fused projection's rows ``[q | k | v]`` (its float32 sums, or rounded already; ``q`` alone for
+    a run that stores nothing) get their ``bias`` (float32, a row's length, or None) and are rounded
+    once to ``out_dtype``: ``q`` is returned as ``[tokens, q_size]``, keys and values go to the tokens'
+    cache slots (values transposed inside their page with ``v_transposed``)."""
+    if proj.dim() != 2 or proj.stride(1) != 1:
+        raise KernelError("qkv_bias_store takes a 2-D projection")
+    tokens, row = proj.shape
+    need = q_size + (k_size + v_size if store else 0)
+    if row < need or (bias is not None and bias.numel() < need):
+        raise KernelError("qkv_bias_store: the projection's rows or the bias are too short")
+    page_size = 0
+    if store:
+        if k_cache is None or v_cache is None or slot_map is None or slot_map.numel() != tokens:
+            raise KernelError("qkv_bias_store: storing needs the caches and one slot per token")
+        if k_cache.dtype != out_dtype or v_cache.dtype != out_dtype:
+            raise KernelError("qkv_bias_store: the caches are not of the output's type")
+        if k_cache.shape[2] * k_cache.shape[3] != k_size or v_cache.numel() != k_cache.shape[0] * k_cache.shape[1] * v_size:
+            raise KernelError("qkv_bias_store: the caches do not match the sizes of k and v")
+        page_size = k_cache.shape[1] if v_transposed else 0
+    q = torch.empty((tokens, q_size), dtype=out_dtype, device=proj.device)
+    _lib.call("pylon_qkv_bias_store", _dev(q, "q"), _dev(k_cache if store else None, "k_cache"),
+              _dev(v_cache if store else None, "v_cache"), dtype_code(out_dtype), proj.data_ptr(),
+              dtype_code(proj.dtype), proj.stride(0), _dev(bias, "bias", torch.float32),
+              _dev(slot_map if store else None, "slot_map", torch.int32), tokens, q_size, k_size, v_size,
+              page_size, 1 if store else 0, _stream())
+    return q
+
+
 def gated_act(gate_up: torch.Tensor, *, alpha: float, offset: float, limit: float,
-              out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+              out_dtype: Optional[torch.dtype] = None, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``a(g) * (u + offset)`` for a ``[tokens, 2I]`` input holding ``g`` then ``u``, with
     ``a(g) = g * sigmoid(alpha * g)``, ``g`` capped from above at ``limit`` and ``u`` to
-    ``[-limit, limit]`` (``limit <= 0``: no cap).  float32 sums in, bfloat16 out: one rounding."""
+    ``[-limit, limit]`` (``limit <= 0``: no cap).  float32 sums in, bfloat16 out: one rounding.
+    ``bias`` (float32 ``[2I]``) is added to ``g`` and ``u`` first."""
     if gate_up.dim() != 2 or gate_up.shape[1] % 2:
         raise KernelError("gated_act takes a [tokens, 2*I] input")
     tokens, two_i = gate_up.shape
+    if bias is not None and bias.shape != (two_i,):
+        raise KernelError("gated_act: one bias per column of the input")
     out = torch.empty((tokens, two_i // 2), dtype=out_dtype or gate_up.dtype, device=gate_up.device)
     _lib.call("pylon_gated_act", _dev(out, "out"), dtype_code(out.dtype), _dev(gate_up, "gate_up"),
-              dtype_code(gate_up.dtype), tokens, two_i // 2, float(alpha), float(offset), float(limit), _stream())
+              dtype_code(gate_up.dtype), tokens, two_i // 2, float(alpha), float(offset), float(limit),
+              _dev(bias, "bias", torch.float32), _stream())
     return out
 
 
@@ -1141,30 +1272,63 @@ def route_top(logits: torch.Tensor, bias: Optional[torch.Tensor], *, n_experts: 
     return experts, weights, gate
 
 
+def route_scored(logits: torch.Tensor, correction: Optional[torch.Tensor], *, n_experts: int, top: int,
+                 groups: int = 1, keep: int = 1, scale: float = 1.0):
+    """From float32 router logits ``[tokens, outputs]``, of which the first ``n_experts`` are experts
+    and the others identity experts: scores are the softmax over all outputs; ``correction`` (float32
+    ``[outputs]``) is added for the choice only; the outputs form ``groups`` equal groups of
+    neighbours, and only the ``keep`` groups with the largest corrected score may be chosen from;
+    the ``top`` largest corrected scores are taken (the lower index among equals).  Returns the
+    chosen outputs (int32 ``[tokens, top]``; an identity keeps its index ``>= n_experts``), their
+    weights ``score * scale`` (float32 ``[tokens, top]``, zero for an identity) and the sum of the
+    chosen identities' weights (float32 ``[tokens]``; None if every output is an expert)."""
+    if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1:
+        raise KernelError("route_scored takes float32 logits [tokens, outputs]")
+    tokens, outputs = logits.shape
+    if correction is not None and correction.shape != (outputs,):
+        raise KernelError("route_scored: one correction per router output")
+    experts = torch.empty((tokens, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((tokens, top), dtype=torch.float32, device=logits.device)
+    identity = torch.empty((tokens,), dtype=torch.float32, device=logits.device) if outputs > n_experts else None
+    _lib.call("pylon_route_scored", _dev(experts, "experts"), _dev(weights, "weights"), _dev(identity, "identity"),
+              logits.data_ptr(), logits.stride(0), _dev(correction, "correction", torch.float32), tokens, outputs,
+              n_experts, top, int(groups), int(keep), float(scale), _stream())
+    return experts, weights, identity
+
+
+EXPERT_ACTS = {"silu_gated": 0, "relu2": 1}  # silu(W_gate x) * (W_up x); relu(W_up x)^2
+
+
 def expert_gate_up(x: torch.Tensor, gate_up: torch.Tensor, experts: torch.Tensor, *, n_experts: int,
-                   ff: int) -> torch.Tensor:
+                   ff: int, act: str = "silu_gated") -> torch.Tensor:
     """``silu(W_gate[e] x_t) * (W_up[e] x_t)`` for every token and each of its chosen experts:
     ``gate_up`` is ``[n_experts * 2 ff, width]`` (an expert's gate rows, then its up rows);
-    returns ``[tokens * top, ff]`` of ``x``'s type, float sums rounded once."""
+    returns ``[tokens * top, ff]`` of ``x``'s type, float sums rounded once.  ``act="relu2"``: plain
+    experts, ``relu(W_up[e] x_t)^2`` with the matrix ``[n_experts * ff, width]``.  A choice of
+    ``n_experts`` or more (an identity) is passed over: its rows of the result are not written."""
     tokens, width = x.shape
     top = experts.shape[1]
-    if gate_up.shape != (n_experts * 2 * ff, width) or gate_up.stride(1) != 1 or x.stride(1) != 1:
-        raise KernelError("expert_gate_up: the experts' matrix must be [experts * 2 ff, width]")
+    per_expert = 2 * ff if act == "silu_gated" else ff
+    if gate_up.shape != (n_experts * per_expert, width) or gate_up.stride(1) != 1 or x.stride(1) != 1:
+        raise KernelError(f"expert_gate_up: the experts' matrix must be [experts * {per_expert}, width]")
     if experts.shape[0] != tokens or experts.dtype != torch.int32 or not experts.is_contiguous():
         raise KernelError("expert_gate_up: experts must be int32 [tokens, top]")
     hidden = torch.empty((tokens * top, ff), dtype=x.dtype, device=x.device)
     _lib.call("pylon_expert_gate_up", _dev(hidden, "hidden"), x.data_ptr(), dtype_code(x.dtype), x.stride(0),
               gate_up.data_ptr(), dtype_code(gate_up.dtype), gate_up.stride(0), _dev(experts, "experts"), tokens, top,
-              ff, width, _stream())
+              ff, width, EXPERT_ACTS[act], n_experts, _stream())
     return hidden
 
 
 def expert_down(hidden: torch.Tensor, down: torch.Tensor, experts: torch.Tensor, weights: torch.Tensor, *,
                 n_experts: int, width: int, shared: Optional[torch.Tensor] = None,
-                shared_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                shared_gate: Optional[torch.Tensor] = None, identity_x: Optional[torch.Tensor] = None,
+                identity_weight: Optional[torch.Tensor] = None) -> torch.Tensor:
     """float32 ``[tokens, width]``: ``sum_s weights[t, s] W_down[e_s] hidden[(t, s)]`` with ``down``
     ``[n_experts * width, ff]``, plus ``shared_gate[t] * shared[t]`` (``shared`` float32
-    ``[tokens, width]``; without the gate it is added as it is)."""
+    ``[tokens, width]``; without the gate it is added as it is), plus ``identity_weight[t] *
+    identity_x[t]`` (the identity experts' share: the token's input, of ``hidden``'s type).  Choices
+    of ``n_experts`` or more are passed over."""
     tokens, top = experts.shape
     ff = hidden.shape[1]
     if hidden.shape[0] != tokens * top or not hidden.is_contiguous():
@@ -1177,11 +1341,18 @@ def expert_down(hidden: torch.Tensor, down: torch.Tensor, experts: torch.Tensor,
         raise KernelError("expert_down: the shared expert's output must be float32 [tokens, width]")
     if shared_gate is not None and (shared is None or shared_gate.numel() != tokens):
         raise KernelError("expert_down: one gate per token, and only with a shared output")
+    if (identity_x is None) != (identity_weight is None):
+        raise KernelError("expert_down: the identities' inputs and weights go together")
+    if identity_x is not None and (identity_x.shape != (tokens, width) or identity_x.dtype != hidden.dtype
+                                   or identity_x.stride(1) != 1 or identity_weight.numel() != tokens):
+        raise KernelError("expert_down: the identities' input must be [tokens, width] of the hidden activations' type")
     out = torch.empty((tokens, width), dtype=torch.float32, device=hidden.device)
     _lib.call("pylon_expert_down", _dev(out, "out"), _dev(hidden, "hidden"), dtype_code(hidden.dtype),
               down.data_ptr(), dtype_code(down.dtype), down.stride(0), _dev(experts, "experts", torch.int32),
               _dev(weights, "weights", torch.float32), _dev(shared, "shared", torch.float32),
-              _dev(shared_gate, "shared_gate", torch.float32), tokens, top, ff, width, _stream())
+              _dev(shared_gate, "shared_gate", torch.float32), tokens, top, ff, width, n_experts,
+              0 if identity_x is None else identity_x.data_ptr(), 0 if identity_x is None else identity_x.stride(0),
+              _dev(identity_weight, "identity_weight", torch.float32), _stream())
     return out
 
 
@@ -1199,19 +1370,23 @@ def experts_grouped_ok(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tenso
 
 def experts_grouped(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, experts: torch.Tensor,
                     weights: torch.Tensor, *, n_experts: int, ff: int, shared: Optional[torch.Tensor] = None,
-                    shared_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    shared_gate: Optional[torch.Tensor] = None, act: str = "silu_gated",
+                    identity_weight: Optional[torch.Tensor] = None) -> torch.Tensor:
     """What :func:`expert_gate_up` and :func:`expert_down` compute, for many bfloat16 tokens: the
     (token, choice) pairs are sorted by expert on the device (nothing is read back), every expert's
     pairs go through its gate/up and its down matrix as tiles of 64 rows on the matrix cores, and
     the results return to their tokens weighted, in the order of the token's choices.  float32
-    ``[tokens, width]``."""
+    ``[tokens, width]``.  ``act`` as for :func:`expert_gate_up`.  Choices of ``n_experts`` or more
+    (identity experts) sort behind every expert's pairs and run through no matrix; with
+    ``identity_weight`` (float32 ``[tokens]``) ``identity_weight[t] * x[t]`` is added for them."""
     tokens, width = x.shape
     top = experts.shape[1]
     pairs = tokens * top
     if not experts_grouped_ok(x, gate_up, down):
         raise KernelError("experts_grouped does not take these operands")
-    if gate_up.shape != (n_experts * 2 * ff, width) or down.shape != (n_experts * width, ff):
-        raise KernelError("experts_grouped: the experts' matrices must be [experts * 2 ff, width] and [experts * width, ff]")
+    per_expert = 2 * ff if act == "silu_gated" else ff
+    if gate_up.shape != (n_experts * per_expert, width) or down.shape != (n_experts * width, ff):
+        raise KernelError(f"experts_grouped: the experts' matrices must be [experts * {per_expert}, width] and [experts * width, ff]")
     flat = experts.reshape(-1).long()
     order = torch.argsort(flat, stable=True)  # sorted place -> pair
     bounds = torch.arange(n_experts + 1, device=x.device)
@@ -1221,14 +1396,17 @@ def experts_grouped(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, 
     hidden = torch.empty((pairs, ff), dtype=torch.bfloat16, device=x.device)
     _lib.call("pylon_grouped_gate_up", _dev(hidden, "hidden"), x.data_ptr(), x.stride(0), _dev(rows, "rows"),
               gate_up.data_ptr(), gate_up.stride(0), _dev(offsets, "offsets"), pairs, n_experts, ff, width, tokens,
-              _stream())
+              EXPERT_ACTS[act], _stream())
     y = torch.empty((pairs, width), dtype=torch.float32, device=x.device)
     _lib.call("pylon_grouped_down", _dev(y, "y"), _dev(hidden, "hidden"), ff, down.data_ptr(), down.stride(0),
               _dev(offsets, "offsets"), pairs, n_experts, ff, width, _stream())
     out = torch.empty((tokens, width), dtype=torch.float32, device=x.device)
     _lib.call("pylon_expert_combine", _dev(out, "out"), _dev(y, "y"), _dev(place, "place"),
               _dev(weights, "weights", torch.float32), _dev(shared, "shared", torch.float32),
-              _dev(shared_gate, "shared_gate", torch.float32), tokens, top, width, _stream())
+              _dev(shared_gate, "shared_gate", torch.float32), tokens, top, width,
+              offsets[n_experts:].data_ptr(),  # where the identities' pairs begin
+              0 if identity_weight is None else x.data_ptr(), 0 if identity_weight is None else x.stride(0),
+              _dev(identity_weight, "identity_weight", torch.float32), _stream())
     return out
 
 

@@ -1,6 +1,6 @@
 """The parts layers are assembled from; importing this package registers the built-in ones."""
 from . import attention, block, feed_forward, latent_attention, logits, mixture, norm, position, retention, short_conv  # noqa: F401
-from .base import KVRequirement, Normed, Part, StateRequirement, requirement_list, summed
+from .base import DepthMixed, KVRequirement, Normed, Part, Scaled, StateRequirement, requirement_list, summed
 from .registry import build_part, register_part, registered, unregister_part
 
 __all__ = [
@@ -8,6 +8,8 @@ __all__ = [
     "StateRequirement",
     "Part",
     "Normed",
+    "Scaled",
+    "DepthMixed",
     "requirement_list",
     "summed",
     "build_part",

@@ -190,7 +190,15 @@ class SinkAttention(Part):
     values transposed inside their page (slot in page fastest), which is how the matrix-core
     kernel reads them; scores, bias and softmax are float32.  bfloat16 steps over pages of a
     multiple of 32 tokens run on the matrix cores (prompt portions as tiles of up to 32 tokens,
-    a step of single tokens as one tile a token); everything else on the general kernel."""
+    a step of single tokens as one tile a token); everything else on the general kernel.
+
+    The spec may ask instead for a bias that grows with the logarithm of the distance and is taken
+    off the score, ``a_h * log(1 + b_h * (i - j))`` with two learned numbers per head
+    (``bias_form="log"``; while a window or chunks bound the distances it reaches the matrix-core
+    kernel as the same table by distance, computed once in float32); for keys visible inside the
+    query's chunk of positions or a window only; for biases of the q, k and v projections (added to
+    the product's float32 sums, rounded once, in the kernel that stores k and v); and for a layer
+    that only ever runs on another run's keys and values (``own_kv`` False: q projection alone)."""
 
     def __init__(self, spec: SinkAttentionSpec, *, dtype: torch.dtype, device) -> None:
         super().__init__()
@@ -201,53 +209,89 @@ class SinkAttention(Part):
                              "both take 1 to 512")
         if spec.window is not None and spec.window < 1:
             raise ValueError("window must be positive (or None for full attention)")
+        if spec.chunk is not None and (spec.chunk < 1 or spec.window is not None):
+            raise ValueError("chunk must be positive, and a layer has a window or chunks, not both")
+        if spec.bias_form not in ("table", "log"):
+            raise ValueError(f"bias_form must be 'table' or 'log', got {spec.bias_form!r}")
         self.spec = spec
         self.dtype = dtype
         self.q_size = spec.n_heads * spec.head_dim
         self.k_size = spec.n_kv_heads * spec.head_dim
         self.v_size = spec.n_kv_heads * spec.v_head_dim
-        self.add_param("qkv", (self.q_size + self.k_size + self.v_size, spec.hidden_size), dtype, device)
+        rows = self.q_size + (self.k_size + self.v_size if spec.own_kv else 0)
+        self.add_param("qkv", (rows, spec.hidden_size), dtype, device)
+        if spec.qkv_bias:
+            self.add_param("qkv_bias", (rows,), torch.float32, device, role="vector")
         self.add_param("out", (spec.hidden_size, spec.n_heads * spec.v_head_dim), dtype, device)
-        self.add_param("rel", (spec.bias_rows, spec.n_heads), torch.float32, device, role="vector")
-        self.bucket = torch.tensor(distance_buckets(spec.bias_rows, spec.bias_far), dtype=torch.int32).to(device)
-        self._bias = None  # (version of rel, the table looked up by distance)
+        self.span = spec.window if spec.window is not None else spec.chunk  # the most keys a token sees (None: all)
+        if spec.bias_form == "table":
+            self.add_param("rel", (spec.bias_rows, spec.n_heads), torch.float32, device, role="vector")
+            self.bucket = torch.tensor(distance_buckets(spec.bias_rows, spec.bias_far), dtype=torch.int32).to(device)
+            self.bias_len = self.bucket.numel()
+        else:
+            # per head the factor a, then per head the slope b
+            self.add_param("log_bias", (2 * spec.n_heads,), torch.float32, device, role="vector")
+            self.bucket = None
+            # as a table by distance it has one entry per distance a token can look back over
+            self.bias_len = self.span if self.span is not None else ops.SINK_MAX_BIAS + 1
+        self._bias = None  # (version of the parameter, the table by distance)
 
     def bias_by_distance(self) -> torch.Tensor:
-        """``rel`` looked up for every distance once, [heads, distances]; made anew when the
-        parameter has been written since (a load, random weights drawn in place)."""
-        rel = self.params["rel"]
-        key = (rel.data_ptr(), rel._version)
+        """The bias of every distance, float32 [heads, distances]: ``rel`` looked up, or ``-a log(1 + b
+        d)`` evaluated, once; made anew when the parameter has been written since (a load, random
+        weights drawn in place)."""
+        source = self.params["rel"] if self.spec.bias_form == "table" else self.params["log_bias"]
+        key = (source.data_ptr(), source._version)
         if self._bias is None or self._bias[0] != key:
-            self._bias = (key, ops.bias_by_distance(rel, self.bucket))
+            if self.spec.bias_form == "table":
+                table = ops.bias_by_distance(source, self.bucket)
+            else:
+                a, b = source.view(2, self.spec.n_heads, 1)
+                distance = torch.arange(self.bias_len, dtype=torch.float32, device=source.device)
+                table = (-a * torch.log(1.0 + b * distance)).contiguous()
+            self._bias = (key, table)
         return self._bias[1]
 
     def cache_requirement(self) -> KVRequirement:
         spec = self.spec
-        return KVRequirement(spec.n_kv_heads, spec.head_dim, spec.window, v_head_dim=spec.v_head_dim)
+        if not spec.cache_bounded:
+            return KVRequirement(spec.n_kv_heads, spec.head_dim, None, v_head_dim=spec.v_head_dim)
+        return KVRequirement(spec.n_kv_heads, spec.head_dim, spec.window, v_head_dim=spec.v_head_dim, chunk=spec.chunk)
 
     def _matrix_cores(self, page_size: int) -> bool:
         spec = self.spec
         return ops.attention_sink_ok(self.dtype, head_dim=spec.head_dim, v_dim=spec.v_head_dim, page_size=page_size,
-                                     bucket_len=self.bucket.numel(), window=spec.window)
+                                     bucket_len=self.bias_len)
 
     def decode_signature(self, rows: int, bound: int) -> tuple:
         """Of a bound on the lengths a step of single tokens takes only over how many workgroups
         a request's keys are cut."""
         if self.dtype != torch.bfloat16:
             return ("sink_attention",)
-        return ("sink_attention", ops.sink_cuts(rows, self.spec.n_heads, self.spec.n_kv_heads, bound))
+        span = bound if self.span is None else min(bound, self.span)
+        return ("sink_attention", ops.sink_cuts(rows, self.spec.n_heads, self.spec.n_kv_heads, span))
 
     def forward(self, h: torch.Tensor, ctx, cache, stores: bool) -> torch.Tensor:
         spec = self.spec
         tokens = h.shape[0]
+        if stores and not spec.own_kv:
+            raise ValueError("a layer without k and v projections can only run on another run's keys and values")
         weight = self.params["qkv"] if stores else self.params["qkv"][: self.q_size]
-        qkv = ops.linear(h, weight, out_dtype=self.dtype)
         pages, page_size = cache.v.shape[0], cache.page_size
         v_cache = cache.v.view(pages, spec.n_kv_heads, spec.v_head_dim, page_size)
-        if stores:
-            ops.kv_store(qkv, cache.k, v_cache, cache.slot_map, k_off=self.q_size, v_off=self.q_size + self.k_size,
-                         v_transposed=True)
+        if spec.qkv_bias:
+            # the biases join the product's float32 sums; q, k and v are rounded once
+            sums = ops.linear(h, weight, out_dtype=torch.float32)
+            qkv = ops.qkv_bias_store(sums, self.params["qkv_bias"], cache.k, v_cache, cache.slot_map,
+                                     q_size=self.q_size, k_size=self.k_size, v_size=self.v_size, out_dtype=self.dtype,
+                                     store=stores, v_transposed=True)
+        else:
+            qkv = ops.linear(h, weight, out_dtype=self.dtype)
+            if stores:
+                ops.kv_store(qkv, cache.k, v_cache, cache.slot_map, k_off=self.q_size,
+                             v_off=self.q_size + self.k_size, v_transposed=True)
         q = qkv.as_strided((tokens, spec.n_heads, spec.head_dim), (qkv.stride(0), spec.head_dim, 1))
+        mask = dict(window=spec.window, chunk=spec.chunk)
         if self._matrix_cores(page_size) and qkv.stride(0) % 8 == 0:
             # tiles heaviest first (turning every second run of the order round, as the plain prefill
             # kernel's caller does, loses here: 227 -> 270 us a layer at 2,048 tokens with four waves a
@@ -255,15 +299,21 @@ class SinkAttention(Part):
             tiles = None if ctx.decode_only else ctx.token_tiles(ops.SINK_TILE)
             # a prompt portion's tiles keep their keys whole: cut in two or four, with the merge behind,
             # a 2,048-token prompt of eight layers took 6.18 and 6.58 ms against 5.82
-            cuts = ops.sink_cuts(tokens, spec.n_heads, spec.n_kv_heads, ctx.max_len) if ctx.decode_only else 1
+            span = ctx.max_len if self.span is None else min(ctx.max_len, self.span)
+            cuts = ops.sink_cuts(tokens, spec.n_heads, spec.n_kv_heads, span) if ctx.decode_only else 1
             context = ops.attention_sink(q, cache.k, v_cache, cache.block_table, tiles, ctx.positions,
                                          page_size=page_size, scale=spec.scale, bias=self.bias_by_distance(),
-                                         sink=spec.sink, cuts=cuts)
+                                         sink=spec.sink, cuts=cuts, **mask)
+        elif spec.bias_form == "table":
+            context = ops.paged_attention(
+                q, cache.k, v_cache, cache.block_table, ctx.tok_row, ctx.positions, page_size=page_size,
+                scale=spec.scale, rel=self.params["rel"], bucket=self.bucket, sink=spec.sink,
+                v_transposed=True, **mask)
         else:
             context = ops.paged_attention(
                 q, cache.k, v_cache, cache.block_table, ctx.tok_row, ctx.positions, page_size=page_size,
-                window=spec.window, scale=spec.scale, rel=self.params["rel"], bucket=self.bucket, sink=spec.sink,
-                v_transposed=True)
+                scale=spec.scale, log_bias=self.params["log_bias"].view(2, spec.n_heads), sink=spec.sink,
+                v_transposed=True, **mask)
         return ops.linear_for_residual(context.view(tokens, spec.n_heads * spec.v_head_dim), self.params["out"],
                                        out_dtype=self.dtype)
 

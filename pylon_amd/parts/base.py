@@ -115,6 +115,28 @@ class Normed:
     eps: float
 
 
+@dataclass
+class Scaled:
+    """A part's output that is still to get a ``bias`` per element (a projection's bias that was left
+    for the sum), to be multiplied element by element by ``scale`` and added to the residual stream
+    (either may be None).  ``value`` as in :class:`Normed`."""
+
+    value: torch.Tensor
+    scale: Optional[torch.Tensor] = None
+    bias: Optional[torch.Tensor] = None
+
+
+@dataclass
+class DepthMixed(Scaled):
+    """As :class:`Scaled`, and once it is added the sum is a layer's result: it becomes
+    ``streams[index]`` (float32 ``[total, tokens, dim]``, one stream per layer so far and the embedded
+    tokens first), and the residual stream is replaced by ``sum_{j <= index} coeff[j] * streams[j]``."""
+
+    streams: Optional[torch.Tensor] = None
+    index: int = 0
+    coeff: Optional[torch.Tensor] = None
+
+
 def summed(delta: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
     """A part's output that has not been added to the residual stream yet, as one float32
     ``[tokens, dim]`` tensor.  What a mixer or a feed-forward hands on is either a tensor of
@@ -128,6 +150,14 @@ def summed(delta: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
         value = summed(delta.value)
         rms = torch.sqrt(value.square().mean(dim=-1, keepdim=True) + delta.eps)
         return value / rms * delta.gain.float()
+    if isinstance(delta, DepthMixed):
+        raise TypeError("a layer's result that is mixed with the earlier layers' needs a norm that knows how "
+                        "(the built-in rmsnorm does)")
+    if isinstance(delta, Scaled):
+        value = summed(delta.value)
+        if delta.bias is not None:
+            value = value + delta.bias.float()
+        return value if delta.scale is None else value * delta.scale.float()
     return delta.sum(dim=0) if delta.dim() == 3 else delta.float()
 
 

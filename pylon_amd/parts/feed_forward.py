@@ -21,10 +21,31 @@ class GatedFeedForward(Part):
         self.add_param("gate_up", (2 * spec.intermediate_size, spec.hidden_size), dtype, device,
                        row_padding=plan.gated_row_padding(spec.hidden_size, element_size))
         self.add_param("down", (spec.hidden_size, spec.intermediate_size), dtype, device)
+        # With biases: those of gate and up enter in the activation kernel, on the product's float32
+        # sums; the down projection's is added here, or, if the block says so, left to the residual sum.
+        self.defer_output_bias = False
+        if spec.bias:
+            self.add_param("gate_up_bias", (2 * spec.intermediate_size,), torch.float32, device, role="vector")
+            self.add_param("down_bias", (spec.hidden_size,), torch.float32, device, role="vector")
+
+    @property
+    def output_bias(self):
+        return self.params.get("down_bias")
 
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
-        hidden = ops.linear_glu(h, self.params["gate_up"], out_dtype=self.dtype)
-        return ops.linear_for_residual(hidden, self.params["down"], out_dtype=self.dtype)
+        if not self.spec.bias:
+            hidden = ops.linear_glu(h, self.params["gate_up"], out_dtype=self.dtype)
+            return ops.linear_for_residual(hidden, self.params["down"], out_dtype=self.dtype)
+        sums = ops.linear(h, self.params["gate_up"], out_dtype=torch.float32)
+        hidden = ops.gated_act(sums, alpha=1.0, offset=0.0, limit=0.0, out_dtype=self.dtype,
+                               bias=self.params["gate_up_bias"])
+        out = ops.linear_for_residual(hidden, self.params["down"], out_dtype=self.dtype)
+        if self.defer_output_bias:
+            return out
+        if out.dim() == 3:  # partial sums: the bias joins the first
+            ops.add_bias_(out[0], self.params["down_bias"])
+            return out
+        return ops.add_bias_(out.float() if out.dtype != torch.float32 else out, self.params["down_bias"])
 
 
 class CappedGatedFeedForward(Part):

@@ -12,6 +12,13 @@ device instead and every expert's pairs run as tiles on the matrix cores).  The 
 product kernels.  The result is float32 and goes to the residual sum unrounded.  A token's
 output does not depend on which other tokens share its step: every kernel here works token by
 token with a fixed order of additions.
+
+The spec may ask instead for plain experts ``down(relu(up(h))^2)`` (``expert_act="relu2"``: one
+matrix ``up`` in place of ``gate_up``), and for the other way of routing (``scoring="softmax_all"``,
+:func:`ops.route_scored`): scores from a softmax over all router outputs, a correction for the choice
+only, a choice limited to the best groups of neighbouring outputs, weights that are the scores times a
+constant, and identity experts (router outputs without matrices, whose output is the input itself:
+the expert kernels pass over them and add the input times the sum of their weights).
 """
 from __future__ import annotations
 
@@ -32,17 +39,38 @@ class MixtureFeedForward(Part):
             raise ValueError("the router kernel takes up to 512 experts and up to 32 of them a token")
         if spec.shared_size is None and spec.shared_gate:
             raise ValueError("a gate of the shared expert needs a shared expert")
+        if spec.expert_act not in ops.EXPERT_ACTS:
+            raise ValueError(f"unknown activation of the experts {spec.expert_act!r} (known: {', '.join(ops.EXPERT_ACTS)})")
+        if spec.scoring not in ("top_softmax", "softmax_all"):
+            raise ValueError(f"unknown scoring {spec.scoring!r} (known: top_softmax, softmax_all)")
+        outputs = spec.n_experts + spec.n_identity
+        if spec.scoring == "top_softmax":
+            if spec.n_identity or spec.groups != 1 or spec.route_scale != 1.0:
+                raise ValueError("identity experts, groups and a scale of the weights belong to the scoring softmax_all")
+        else:
+            if spec.n_identity < 0 or outputs > 512 or spec.top > outputs:
+                raise ValueError(f"the router has 1 to 512 outputs and a token takes at most all of them, not {spec.top} of {outputs}")
+            if spec.groups < 1 or outputs % spec.groups or not 1 <= spec.groups_kept <= spec.groups:
+                raise ValueError(f"{outputs} router outputs do not form {spec.groups} equal groups of which "
+                                 f"{spec.groups_kept} are kept")
+            if spec.shared_gate:
+                raise ValueError("the gate of a shared expert is one more router row of the scoring top_softmax only")
         self.spec = spec
         self.dtype = dtype
+        self.gated = spec.expert_act == "silu_gated"
         width, ff = spec.hidden_size, spec.expert_size
-        self.router_rows = spec.n_experts + (1 if spec.shared_gate else 0)
+        self.router_rows = outputs + (1 if spec.shared_gate else 0)
         # stored in 16 bits it stays so: products of two bfloat16 numbers are exact in float32, and the
         # product kernels add them up in float32 and hand the sums back unrounded
         self.add_param("router", (self.router_rows, width), dtype, device)
         if spec.router_bias:
-            self.add_param("router_bias", (spec.n_experts,), torch.float32, device, role="vector")
+            self.add_param("router_bias", (outputs,), torch.float32, device, role="vector")
         # expert e: rows [e * 2 ff, e * 2 ff + ff) its gate, the next ff its up; rows [e * width, ...) its down
-        self.add_param("gate_up", (spec.n_experts * 2 * ff, width), dtype, device)
+        # (plain experts: rows [e * ff, ...) its up)
+        if self.gated:
+            self.add_param("gate_up", (spec.n_experts * 2 * ff, width), dtype, device)
+        else:
+            self.add_param("up", (spec.n_experts * ff, width), dtype, device)
         self.add_param("down", (spec.n_experts * width, ff), dtype, device)
         if spec.shared_size is not None:
             element_size = torch.empty((), dtype=dtype).element_size()
@@ -53,21 +81,31 @@ class MixtureFeedForward(Part):
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
         spec = self.spec
         logits = ops.linear(h, self.params["router"], out_dtype=torch.float32)
-        experts, weights, shared_gate = ops.route_top(
-            logits, self.params.get("router_bias"), n_experts=spec.n_experts, top=spec.top,
-            shared_gate=spec.shared_gate)
+        identity = None
+        if spec.scoring == "softmax_all":
+            shared_gate = None
+            experts, weights, identity = ops.route_scored(
+                logits, self.params.get("router_bias"), n_experts=spec.n_experts, top=spec.top, groups=spec.groups,
+                keep=spec.groups_kept, scale=spec.route_scale)
+        else:
+            experts, weights, shared_gate = ops.route_top(
+                logits, self.params.get("router_bias"), n_experts=spec.n_experts, top=spec.top,
+                shared_gate=spec.shared_gate)
+        first = self.params["gate_up"] if self.gated else self.params["up"]
         shared = None
         if spec.shared_size is not None:
             shared_hidden = ops.linear_glu(h, self.params["shared_gate_up"], out_dtype=self.dtype)
             shared = ops.linear(shared_hidden, self.params["shared_down"], out_dtype=torch.float32)
-        if h.shape[0] >= ops.GROUPED_FROM and ops.experts_grouped_ok(h, self.params["gate_up"], self.params["down"]):
+        if h.shape[0] >= ops.GROUPED_FROM and ops.experts_grouped_ok(h, first, self.params["down"]):
             # many tokens: sorted by expert, every expert's tokens as tiles on the matrix cores
-            return ops.experts_grouped(h, self.params["gate_up"], self.params["down"], experts, weights,
+            return ops.experts_grouped(h, first, self.params["down"], experts, weights,
                                        n_experts=spec.n_experts, ff=spec.expert_size, shared=shared,
-                                       shared_gate=shared_gate)
-        hidden = ops.expert_gate_up(h, self.params["gate_up"], experts, n_experts=spec.n_experts, ff=spec.expert_size)
+                                       shared_gate=shared_gate, act=spec.expert_act, identity_weight=identity)
+        hidden = ops.expert_gate_up(h, first, experts, n_experts=spec.n_experts, ff=spec.expert_size,
+                                    act=spec.expert_act)
         return ops.expert_down(hidden, self.params["down"], experts, weights, n_experts=spec.n_experts,
-                               width=spec.hidden_size, shared=shared, shared_gate=shared_gate)
+                               width=spec.hidden_size, shared=shared, shared_gate=shared_gate,
+                               identity_x=h if identity is not None else None, identity_weight=identity)
 
 
 register_part("feed_forward", "mixture", MixtureFeedForward, replace=True)

@@ -10,7 +10,7 @@ import torch
 
 from ..config.specs import NormSpec
 from ..kernels import ops
-from .base import Normed, Part
+from .base import DepthMixed, Normed, Part, Scaled
 from .registry import register_part
 
 
@@ -41,6 +41,18 @@ class RMSNorm(Part):
         if isinstance(delta, Normed):
             return ops.add_normed_rmsnorm(resid, delta.value, self.weight(), self.spec.eps, self.dtype,
                                           post_gain=delta.gain, post_eps=delta.eps, row_idx=row_idx)
+        if isinstance(delta, DepthMixed):
+            # the sum, the layer's result among the streams, their mix and its norm in one kernel;
+            # where only some rows are normed, the mix of all rows first
+            fused = row_idx is None
+            out = ops.depth_mix(resid, delta.value, delta.streams, delta.index, delta.coeff, delta_scale=delta.scale,
+                                delta_bias=delta.bias, gain=self.weight() if fused else None, eps=self.spec.eps,
+                                out_dtype=self.dtype)
+            return out if fused else ops.rmsnorm(resid, self.weight(), self.spec.eps, out_dtype=self.dtype,
+                                                 row_idx=row_idx)
+        if isinstance(delta, Scaled):
+            return ops.add_normed_rmsnorm(resid, delta.value, self.weight(), self.spec.eps, self.dtype,
+                                          row_idx=row_idx, delta_scale=delta.scale, delta_bias=delta.bias)
         return ops.add_rmsnorm(resid, delta, self.weight(), self.spec.eps, self.dtype,
                                row_idx=row_idx)
 

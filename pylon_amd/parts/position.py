@@ -14,7 +14,8 @@ from typing import Optional, Tuple
 
 import torch
 
-from ..config.specs import PositionSpec
+from ..config.specs import PositionSpec, SinusoidPositionSpec
+from ..kernels import ops
 from .base import Part
 from .registry import register_part
 
@@ -50,5 +51,24 @@ class NoPosition(Part):
         return None
 
 
+class SinusoidPosition(Part):
+    """A part of the family "stream": a fixed position vector added to the embedded tokens, element
+    ``2i`` the sine and element ``2i + 1`` the cosine of ``position * base**(-2i/dim)``.  The
+    frequencies are formed in double precision and rounded to float32 once; the angle is the float32
+    product of position and frequency."""
+
+    def __init__(self, spec: SinusoidPositionSpec, *, dtype: torch.dtype, device) -> None:
+        super().__init__()
+        if spec.dim < 1 or not spec.base > 0:
+            raise ValueError("a sinusoidal position vector needs a positive size and base")
+        self.spec = spec
+        exponents = torch.arange(0, spec.dim, 2, dtype=torch.float64) / spec.dim
+        self.freq = (torch.tensor(spec.base, dtype=torch.float64) ** -exponents).to(torch.float32).to(device)
+
+    def forward(self, resid: torch.Tensor, ctx) -> torch.Tensor:
+        return ops.add_sinusoid(resid, ctx.positions, self.freq)
+
+
 register_part("position", "rope", RotaryPosition, replace=True)
+register_part("stream", "sinusoid", SinusoidPosition, replace=True)
 register_part("position", "none", NoPosition, replace=True)

@@ -6,7 +6,7 @@ from __future__ import annotations
 
 import torch
 
-from ..config.specs import ShortConvSpec
+from ..config.specs import ShortConvSpec, TokenShiftSpec
 from ..kernels import ops
 from .base import Part, StateRequirement
 from .registry import register_part
@@ -34,4 +34,26 @@ class ShortConv(Part):
                               max_count=ctx.max_count, out_dtype=self.dtype)
 
 
+class TokenShift(Part):
+    """``h + (h' - h) * w`` with ``h'`` the previous token's ``h`` (zeros before a request's first
+    token) and ``w`` one learned number per channel, in float32 and rounded once.  A request's last
+    input is state of fixed size in its state slot, so a request can arrive in portions of any size."""
+
+    STATE = "shift"
+
+    def __init__(self, spec: TokenShiftSpec, *, dtype: torch.dtype, device) -> None:
+        super().__init__()
+        self.spec = spec
+        self.dtype = dtype
+        self.add_param("weight", (spec.dim,), torch.float32, device, role="vector")
+
+    def cache_requirement(self):
+        return StateRequirement((self.spec.dim,), torch.float32, name=self.STATE)
+
+    def forward(self, h: torch.Tensor, ctx, cache) -> torch.Tensor:
+        return ops.token_shift(h, self.params["weight"], cache.states[self.STATE], ctx.row_start, ctx.row_slots,
+                               rows=ctx.rows, max_count=ctx.max_count, out_dtype=self.dtype)
+
+
 register_part("conv", "short_conv", ShortConv, replace=True)
+register_part("conv", "token_shift", TokenShift, replace=True)

@@ -34,7 +34,8 @@ def draw_tensor(seed: int, name: str, target, sigma: float, norm_jitter: float, 
     """The one rule of the random-weights mode: fill ``out`` (of the target's shape, on any
     device, of any float type) with tensor ``name`` of seed ``seed``.  ``normal``:
     N(0, sigma^2); ``ones`` / ``ones_jitter``: 1, or 1 + norm_jitter * N(0, 1); ``zeros_jitter``: 0, or
-    norm_jitter * N(0, 1).  The numbers
+    norm_jitter * N(0, 1); ``positive``: 0.05 + |N(0, 1)| / 2 whatever sigma (numbers that must be
+    positive: the slope of a logarithmic bias by distance).  The numbers
     come from a generator keyed by (seed, name) on the device ``draw_on`` (default: where
     ``out`` lives): drawn on the CPU they are the numbers of the folder that
     :func:`write_random_model` writes; drawn on a GPU they follow the same rule with other
@@ -47,12 +48,15 @@ def draw_tensor(seed: int, name: str, target, sigma: float, norm_jitter: float, 
     if target.init == "zeros_jitter" and not norm_jitter:  # a norm weight stored as its distance from one
         out.fill_(0.0)
         return
-    if target.init not in ("normal", "ones_jitter", "zeros_jitter"):
+    if target.init not in ("normal", "ones_jitter", "zeros_jitter", "positive"):
         raise ValueError(f"unknown init rule {target.init!r} for {name}")
     where = torch.device(draw_on) if draw_on is not None else out.device
     gen = _generator(seed, name, where)
-    scale, shift = {"normal": (sigma, 0.0), "ones_jitter": (norm_jitter, 1.0), "zeros_jitter": (norm_jitter, 0.0)}[
-        target.init]
+    scale, shift = {"normal": (sigma, 0.0), "ones_jitter": (norm_jitter, 1.0), "zeros_jitter": (norm_jitter, 0.0),
+                    "positive": (0.5, 0.05)}[target.init]
+    if target.init == "positive":
+        out.copy_(torch.randn(tuple(out.shape), generator=gen, dtype=torch.float32, device=where).abs() * scale + shift)
+        return
     if out.is_contiguous():
         flat = out.view(-1)
         for start in range(0, flat.numel(), _SLAB):
