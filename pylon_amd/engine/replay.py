@@ -22,7 +22,7 @@ from pathlib import Path
 from typing import Dict
 
 PAGE_SIZE = 64  # default page: pool pages are counted in units of 64 tokens, as --max-tokens is
-MAX_LIVE = 8  # default number of state slots (requests live at a time)
+MAX_LIVE = 4  # default number of state slots (requests live at a time)
 
 
 def _note(text: str) -> None:
