@@ -33,8 +33,9 @@ from .registry import register_part
 class MixtureFeedForward(Part):
     def __init__(self, spec: MixtureFeedForwardSpec, *, dtype: torch.dtype, device) -> None:
         super().__init__()
-        if not 1 <= spec.top <= spec.n_experts:
-            raise ValueError(f"a token uses 1 to {spec.n_experts} of {spec.n_experts} experts, not {spec.top}")
+        choices = spec.n_experts + (spec.n_identity if spec.scoring == "softmax_all" else 0)
+        if spec.n_experts < 1 or not 1 <= spec.top <= choices:
+            raise ValueError(f"a token uses 1 to {choices} of {choices} experts, not {spec.top}")
         if spec.n_experts > 512 or spec.top > 32:
             raise ValueError("the router kernel takes up to 512 experts and up to 32 of them a token")
         if spec.shared_size is None and spec.shared_gate:

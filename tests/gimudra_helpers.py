@@ -57,12 +57,13 @@ GIMUDRA_Q = {
 }
 # R: one key/value head for all heads, a layer without any mask (every earlier key: the bias by
 # distance is then evaluated in the kernel), chunks longer than any prompt, more identity experts
-# than experts, groups of one output each, all of them kept.
+# than experts and more of them taken by a token than there are experts, groups of one output each,
+# all of them kept.
 GIMUDRA_R = {
     "architecture": "Gimudra", "vocab": 97, "width": 48, "norm": {"eps": 3e-6}, "embedding": {"scale": 0.25},
     "layers": [
         _layer(_attention(5, 1, 16, 8, 0.25), _dense(20)),
-        _layer(_attention(2, 2, 8, 12, 0.35, 1000), _moe(2, 3, 2, 12, 5, 5, 3.0)),
+        _layer(_attention(2, 2, 8, 12, 0.35, 1000), _moe(2, 3, 3, 12, 5, 5, 3.0)),
     ],
 }
 # S: sizes for the matrix-core kernels over pages of 64, sixteen query heads on one key/value head
