@@ -2,7 +2,7 @@
 and uniform-random token ids, on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
-                    [--shape 4b|8b|32b] [--prompt-len N] [--design vupuzen|pavitar [--design-shapes 8b,...]]
+                    [--shape 4b|8b|32b] [--prompt-len N] [--design vupuzen|pavitar|gimudra [--beside qwen3|vupuzen|pavitar] [--design-shapes 8b,...]]
 
 Everything goes the product's own way.  Start-up is ``Runner.from_random``: the fit check,
 the measured activation headroom, the page pool sized from the card's memory and the decode
@@ -332,6 +332,29 @@ def pavitar_json(shape: dict, layers: int) -> dict:
             "layers": [attention if i % 4 == 0 else latent for i in range(own)]}
 
 
+def gimudra_json(shape: dict, layers: int) -> dict:
+    """A Gimudra configuration of the shape's layer sizes: attention with the shape's heads, equal key
+    and value sizes and chunks of 1,024 positions; of every four layers the first two have keys and
+    values of their own and the other two read the second's; the first of the four has the shape's dense
+    feed-forward, the others a mixture of 28 plain experts and 4 identity experts in 4 groups of which 2
+    are kept, 4 a token, sized so that four experts are as large as the dense feed-forward; the shape's
+    vocabulary."""
+    width, hd = shape["hidden_size"], shape["head_dim"]
+    expert = max(64, shape["intermediate_size"] * 3 // 8 // 64 * 64)
+    moe = {"kind": "moe", "expert": {"ff": expert},
+           "router": {"experts": 28, "identity": 4, "top": 4, "scale": 1.0, "groups": {"count": 4, "keep": 2}}}
+    dense = {"kind": "dense", "ff": shape["intermediate_size"]}
+    out = []
+    for i in range(layers):
+        mixer = {"heads": shape["num_attention_heads"], "kv_heads": shape["num_key_value_heads"], "dim": hd, "vdim": hd,
+                 "scale": hd ** -0.5, "mask": {"size": 1024}}
+        if i % 4 >= 2:
+            mixer["kv_from"] = i - i % 4 + 1
+        out.append({"type": "attention", "mixer": mixer, "mlp": dense if i % 4 == 0 else moe})
+    return {"architecture": "Gimudra", "vocab": shape["vocab_size"], "width": width, "norm": {"eps": 1e-6},
+            "embedding": {"scale": 1.0}, "layers": out}
+
+
 def design_steps(runner, vocab: int, batch: int, prompt_len: int, steps: int, warmup: int, seed: int) -> dict:
     """Milliseconds of one prompt step of ``prompt_len`` tokens (median of five), and of a
     decode step of ``batch`` requests behind such prompts (mean of ``steps``), through the step
@@ -373,10 +396,11 @@ def design_steps(runner, vocab: int, batch: int, prompt_len: int, steps: int, wa
 
 
 def design_main(args) -> int:
-    """``--design vupuzen|pavitar``: prefill and decode of models of that design of random weights
-    at the layer sizes of ``--shape`` (and of the other shapes named by ``--design-shapes``),
-    beside the Qwen3 model of the same sizes and number of layer runs, both through the same step
-    function over pages of 256 tokens with decode graphs."""
+    """``--design vupuzen|pavitar|gimudra``: prefill and decode of models of that design of random
+    weights at the layer sizes of ``--shape`` (and of the other shapes named by ``--design-shapes``),
+    beside the model of the design ``--beside`` (Qwen3 unless told otherwise) of the same sizes and
+    number of layer runs, both through the same step function over pages of 256 tokens with decode
+    graphs."""
     import torch
 
     from pylon_amd.config import PylonConfig
@@ -386,12 +410,15 @@ def design_main(args) -> int:
     points = {}
     prompt_len = args.prompt_len if args.prompt_len != PROMPT_LEN else PREFILL_TOKENS
     steps, warmup = min(args.steps, 128), min(args.warmup, 16)
+    beside = args.beside
+    if beside == args.design:
+        raise SystemExit("--beside names another design than --design")
     for name in [args.shape] + [n for n in (args.design_shapes or "").split(",") if n and n != args.shape]:
         shape = SHAPES[name]
         layers = args.layers or 8
         pages = (args.batch + 1) * (-(-(prompt_len + steps + warmup + 8) // PAGE_SIZE) + 1)
-        mine_json = vupuzen_json(shape, layers) if args.design == "vupuzen" else pavitar_json(shape, layers)
-        for design, raw in ((args.design, mine_json), ("qwen3", config_json(shape, layers))):
+        makers = {"vupuzen": vupuzen_json, "pavitar": pavitar_json, "gimudra": gimudra_json, "qwen3": config_json}
+        for design, raw in ((args.design, makers[args.design](shape, layers)), (beside, makers[beside](shape, layers))):
             config = PylonConfig(dtype=args.dtype, max_batch_size=args.batch + 1, max_queue_size=args.batch + 1,
                                  page_size=PAGE_SIZE, prefill_chunk_size=prompt_len, num_pages=pages,
                                  cuda_graphs=not args.no_graphs)
@@ -401,7 +428,7 @@ def design_main(args) -> int:
             points[f"{design}_{name}"] = point
             del runner
             torch.cuda.empty_cache()
-        mine, theirs = points[f"{args.design}_{name}"], points[f"qwen3_{name}"]
+        mine, theirs = points[f"{args.design}_{name}"], points[f"{beside}_{name}"]
         points[f"ratio_{name}"] = {"prefill": round(mine["prefill_tokens_per_s"] / theirs["prefill_tokens_per_s"], 3),
                                    "decode": round(mine["decode_tokens_per_s"] / theirs["decode_tokens_per_s"], 3)}
         if record is None:
@@ -411,7 +438,7 @@ def design_main(args) -> int:
                 "value": mine["decode_tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
                 "ms_per_step": mine["decode_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
                 "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
-                "config": {"model": f"{args.design}-{name}-sizes-random", "layers": layers, "global_batch": args.batch,
+                "config": {"model": f"{args.design}-{name}-sizes-random", "beside": beside, "layers": layers, "global_batch": args.batch,
                            "seq_len": prompt_len, "page_size": PAGE_SIZE, "hip_graphs": not args.no_graphs,
                            "parallelism": "single-gpu"},
             }
@@ -441,8 +468,10 @@ def main() -> int:
     parser.add_argument("--no-peaks", action="store_true", help="skip the probes of this device's own peaks")
     parser.add_argument("--mixed", action="store_true",
                         help="also time a step of --batch decoded tokens beside a 2,048-token prompt portion")
-    parser.add_argument("--design", choices=("qwen3", "vupuzen", "pavitar"), default="qwen3",
-                        help="vupuzen, pavitar: that design beside Qwen3 at equal sizes instead of the default workload")
+    parser.add_argument("--design", choices=("qwen3", "vupuzen", "pavitar", "gimudra"), default="qwen3",
+                        help="vupuzen, pavitar, gimudra: that design beside Qwen3 at equal sizes instead of the default workload")
+    parser.add_argument("--beside", choices=("qwen3", "vupuzen", "pavitar"), default="qwen3",
+                        help="with another --design: the design it is measured beside (default qwen3)")
     parser.add_argument("--design-shapes", default="", help="with another --design: further shapes, with commas")
     parser.add_argument("--prefill-only", action="store_true",
                         help="only the prefill measurement (for profiling); prints its part of the record")

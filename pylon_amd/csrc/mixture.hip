@@ -301,6 +301,59 @@ __device__ __forceinline__ void rows_dot_share(const bf16_t* const (&rows)[ROWS]
   }
 }
 
+// The same two with the vector in LDS as bfloat16 as well (half the room, so more workgroups share a
+// unit's LDS, and one LDS read per eight elements): products and order of additions are those of the
+// float versions, so the results are the same to the bit.
+__device__ __forceinline__ float row_dot_share_packed(const bf16_t* __restrict__ row, const bf16_t* __restrict__ xs, int n,
+                                                      int lane, bool wide) {
+  float acc = 0.f;
+  if (wide) {
+    for (int i = lane * 8; i < n; i += PYLON_WAVE * 8) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(row + i);
+      const uint4 xr = *reinterpret_cast<const uint4*>(xs + i);
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+      const uint32_t x[4] = {xr.x, xr.y, xr.z, xr.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc = fmaf(__uint_as_float(x[j] << 16), __uint_as_float(w[j] << 16), acc);
+        acc = fmaf(__uint_as_float(x[j] & 0xffff0000u), __uint_as_float(w[j] & 0xffff0000u), acc);
+      }
+    }
+  } else {
+    for (int i = lane; i < n; i += PYLON_WAVE) acc = fmaf(to_float(xs[i]), to_float(row[i]), acc);
+  }
+  return acc;
+}
+
+template <int ROWS, int PIECES>
+__device__ __forceinline__ void rows_dot_share_packed(const bf16_t* const (&rows)[ROWS], const bf16_t* __restrict__ xs,
+                                                      int n, int lane, float (&acc)[ROWS]) {
+  constexpr int STEP = PYLON_WAVE * 8;
+  for (int i = lane * 8; i < n; i += PIECES * STEP) {
+    uint4 raw[ROWS][PIECES];
+#pragma unroll
+    for (int q = 0; q < ROWS; ++q)
+#pragma unroll
+      for (int p = 0; p < PIECES; ++p)
+        raw[q][p] = i + p * STEP < n ? *reinterpret_cast<const uint4*>(rows[q] + i + p * STEP) : uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int p = 0; p < PIECES; ++p) {
+      if (i + p * STEP >= n) continue;
+      const uint4 xr = *reinterpret_cast<const uint4*>(xs + i + p * STEP);
+      const uint32_t x[4] = {xr.x, xr.y, xr.z, xr.w};
+#pragma unroll
+      for (int q = 0; q < ROWS; ++q) {
+        const uint32_t w[4] = {raw[q][p].x, raw[q][p].y, raw[q][p].z, raw[q][p].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[q] = fmaf(__uint_as_float(x[j] << 16), __uint_as_float(w[j] << 16), acc[q]);
+          acc[q] = fmaf(__uint_as_float(x[j] & 0xffff0000u), __uint_as_float(w[j] & 0xffff0000u), acc[q]);
+        }
+      }
+    }
+  }
+}
+
 template <typename T>
 struct is_bf16 {
   static constexpr bool value = false;
@@ -430,13 +483,24 @@ expert_down_kernel(float* __restrict__ out, const TH* __restrict__ hidden, const
                    const float* __restrict__ shared, const float* __restrict__ shared_gate, int top, int ff,
                    int width, int cols_per_block, int wide, int n_experts, const TH* __restrict__ ident_x,
                    long long ident_stride, const float* __restrict__ ident_w) {
-  extern __shared__ float hs[];  // [top, ff]: the token's hidden activations of its chosen experts
+  // [top, ff]: the token's hidden activations of its chosen experts; bfloat16 activations for
+  // bfloat16 weights stay packed (half the room: twice the workgroups a unit holds), else float
+  constexpr bool PACKED = is_bf16<TH>::value && is_bf16<TW>::value;
+  extern __shared__ __attribute__((aligned(16))) unsigned char hs_raw[];
+  float* hs = reinterpret_cast<float*>(hs_raw);
+  bf16_t* hp = reinterpret_cast<bf16_t*>(hs_raw);
   const int t = blockIdx.y;
   const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
   for (int i = threadIdx.x; i < top * ff; i += 256) {
     // an identity's rows of hidden were never written
     const bool real = experts[static_cast<size_t>(t) * top + i / ff] < n_experts;
-    hs[i] = real ? to_float(hidden[static_cast<size_t>(t) * top * ff + i]) : 0.f;
+    if constexpr (PACKED) {
+      bf16_t v;
+      v.bits = real ? reinterpret_cast<const bf16_t*>(hidden)[static_cast<size_t>(t) * top * ff + i].bits : uint16_t(0);
+      hp[i] = v;
+    } else {
+      hs[i] = real ? to_float(hidden[static_cast<size_t>(t) * top * ff + i]) : 0.f;
+    }
   }
   __syncthreads();
   // identity experts: the token's input itself, times the sum of their weights
@@ -460,7 +524,8 @@ expert_down_kernel(float* __restrict__ out, const TH* __restrict__ hidden, const
 #pragma unroll
         for (int q = 0; q < 4; ++q) rows[q] = base + static_cast<size_t>(c + q < c1 ? c + q : c1 - 1) * w_stride;
         float part[4] = {0.f, 0.f, 0.f, 0.f};
-        rows_dot_share<4, 2>(rows, hs + s * ff, ff, lane, part);
+        if constexpr (PACKED) rows_dot_share_packed<4, 2>(rows, hp + s * ff, ff, lane, part);
+        else rows_dot_share<4, 2>(rows, hs + s * ff, ff, lane, part);
         const float weight = weights[static_cast<size_t>(t) * top + s];
 #pragma unroll
         for (int q = 0; q < 4; ++q) share[q] = fmaf(weight, part[q], share[q]);
@@ -488,7 +553,10 @@ expert_down_kernel(float* __restrict__ out, const TH* __restrict__ hidden, const
       const int e = experts[static_cast<size_t>(t) * top + s];
       if (e >= n_experts) continue;
       const TW* row = w + (static_cast<size_t>(e) * width + c) * w_stride;
-      share = fmaf(weights[static_cast<size_t>(t) * top + s], row_dot_share<TW>(row, hs + s * ff, ff, lane, wide), share);
+      float part;
+      if constexpr (PACKED) part = row_dot_share_packed(reinterpret_cast<const bf16_t*>(row), hp + s * ff, ff, lane, wide);
+      else part = row_dot_share<TW>(row, hs + s * ff, ff, lane, wide);
+      share = fmaf(weights[static_cast<size_t>(t) * top + s], part, share);
     }
     float acc = wave_sum(share);
     if (lane == 0) {
@@ -517,8 +585,10 @@ extern "C" int pylon_expert_down(float* out, const void* hidden, int h_dtype, co
   PYLON_REQUIRE(!(h_dtype == PYLON_F32 && w_dtype == PYLON_BF16), "expert_down: float inputs take float weights");
   PYLON_REQUIRE(tokens >= 0 && top >= 1 && ff >= 1 && width >= 1, "expert_down: sizes must be positive");
   PYLON_REQUIRE(w_stride >= ff, "expert_down: rows overlap");
-  const size_t lds = sizeof(float) * top * ff;
-  PYLON_REQUIRE(lds <= 64 * 1024, "expert_down: %d experts of %d hidden units do not fit LDS", top, ff);
+  const bool packed = h_dtype == PYLON_BF16 && w_dtype == PYLON_BF16;
+  const size_t lds = (packed ? sizeof(uint16_t) : sizeof(float)) * top * ff;
+  // a workgroup of this device may hold 160 KB; beyond 64 KB a kernel has to be told
+  PYLON_REQUIRE(lds <= 160 * 1024, "expert_down: %d experts of %d hidden units do not fit LDS", top, ff);
   if (tokens == 0) return 0;
   const int per = w_dtype == PYLON_F32 ? 4 : 8;
   const int wide = (ff % per == 0 && w_stride % per == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0) ? 1 : 0;
@@ -528,12 +598,17 @@ extern "C" int pylon_expert_down(float* out, const void* hidden, int h_dtype, co
     dim3 grid((width + cols - 1) / cols, n), block(256);
     const size_t off = static_cast<size_t>(first);
 #define GO(TH, TW)                                                                                              \
-  hipLaunchKernelGGL((expert_down_kernel<TH, TW>), grid, block, lds, stream, out + off * width,                 \
-                     (const TH*)hidden + off * top * ff, (const TW*)w, w_stride, experts + off * top,           \
-                     weights + off * top, shared != nullptr ? shared + off * width : nullptr,                   \
-                     shared_gate != nullptr ? shared_gate + off : nullptr, top, ff, width, cols, wide, n_experts, \
-                     ident_x != nullptr ? (const TH*)ident_x + off * ident_stride : nullptr, ident_stride,      \
-                     ident_w != nullptr ? ident_w + off : nullptr)
+  do {                                                                                                          \
+    if (lds > 64 * 1024)                                                                                        \
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&expert_down_kernel<TH, TW>),                     \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));             \
+    hipLaunchKernelGGL((expert_down_kernel<TH, TW>), grid, block, lds, stream, out + off * width,               \
+                       (const TH*)hidden + off * top * ff, (const TW*)w, w_stride, experts + off * top,         \
+                       weights + off * top, shared != nullptr ? shared + off * width : nullptr,                 \
+                       shared_gate != nullptr ? shared_gate + off : nullptr, top, ff, width, cols, wide,        \
+                       n_experts, ident_x != nullptr ? (const TH*)ident_x + off * ident_stride : nullptr,       \
+                       ident_stride, ident_w != nullptr ? ident_w + off : nullptr);                             \
+  } while (0)
     if (h_dtype == PYLON_F32) GO(float, float);
     else if (w_dtype == PYLON_F32) GO(bf16_t, float);
     else GO(bf16_t, bf16_t);

@@ -369,7 +369,8 @@ def test_routing_among_equals_takes_the_lower_index_and_bars_groups_by_their_bes
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("width, experts, identity, top, ff, count, keep", [
     (64, 5, 1, 2, 24, 3, 2), (48, 3, 0, 1, 32, 1, 1), (512, 6, 2, 4, 520, 4, 3), (100, 4, 0, 4, 7, 2, 2),
-    (128, 8, 4, 4, 64, 4, 3), (192, 2, 6, 3, 96, 8, 5), (64, 1, 3, 4, 16, 2, 2)])
+    (128, 8, 4, 4, 64, 4, 3), (192, 2, 6, 3, 96, 8, 5), (64, 1, 3, 4, 16, 2, 2),
+    (128, 6, 2, 4, 4608, 4, 3)])  # the last: a token's hidden activations take more than 64 KB of LDS
 def test_mixture_with_identity_experts_against_the_plain_one(ops, dtype, width, experts, identity, top, ff, count, keep):
     from pylon_amd.config.specs import MixtureFeedForwardSpec
     from pylon_amd.parts import build_part
