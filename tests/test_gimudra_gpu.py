@@ -130,7 +130,7 @@ def test_depth_mix_keeps_every_result_and_hands_on_their_mix(ops, dim, parts, to
     assert np.array_equal(streams[0].cpu().numpy(), first.astype(np.float32))
 
 
-@pytest.mark.parametrize("dim", [6, 192, 5, 1000])
+@pytest.mark.parametrize("dim", [6, 176, 5, 1000])
 def test_position_vectors_of_sines_and_cosines(ops, dim):
     positions = [0, 1, 2, 63, 64, 1000, 4097, 3, 0]
     freq = dev(10000.0 ** (-np.arange(0, dim, 2, dtype=np.float64) / dim))
@@ -170,7 +170,7 @@ def plain_biased_attention(q, k, v, visible, scale, r1, r2):
 @pytest.mark.parametrize("size", [37, 64, 129, 1, 300, None])
 @pytest.mark.parametrize("dtype, heads, groups, dim, vdim, page", [
     (torch.float32, 4, 2, 16, 24, 16), (torch.float32, 3, 1, 12, 20, 16), (torch.bfloat16, 6, 3, 20, 6, 16),
-    (torch.bfloat16, 4, 2, 64, 80, 32), (torch.bfloat16, 8, 2, 64, 80, 64), (torch.bfloat16, 16, 1, 16, 8, 64),
+    (torch.bfloat16, 4, 2, 64, 72, 32), (torch.bfloat16, 8, 4, 64, 48, 64), (torch.bfloat16, 16, 1, 16, 8, 64),
     (torch.bfloat16, 3, 3, 128, 128, 64), (torch.bfloat16, 5, 5, 40, 36, 96)])
 def test_attention_with_a_bias_by_log_distance_at_the_edges_of_chunks_and_pages(ops, size, dtype, heads, groups, dim, vdim, page):
     """Keys planted at both sides of a chunk's edge, at a page's first and last slot and far back;
@@ -263,7 +263,7 @@ def test_a_far_key_among_hundreds_carries_the_output_despite_the_bias(ops):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads, groups, dim, vdim, page, transposed", [(4, 2, 16, 24, 16, True), (3, 1, 12, 20, 32, True),
-                                                                         (8, 2, 64, 80, 64, True), (2, 2, 8, 8, 16, False)])
+                                                                         (6, 2, 64, 72, 64, True), (2, 2, 8, 8, 16, False)])
 def test_biases_join_the_projections_before_the_one_rounding(ops, dtype, heads, groups, dim, vdim, page, transposed):
     rng = np.random.default_rng(dim + vdim)
     n, pages = 45, 5
@@ -318,7 +318,7 @@ def router_of(experts, identity, top, count, keep, scale):
 
 
 @pytest.mark.parametrize("experts, identity, top, count, keep", [
-    (12, 4, 4, 4, 3), (5, 1, 2, 3, 2), (4, 0, 4, 1, 1), (2, 3, 2, 5, 5), (8, 0, 1, 4, 1), (60, 4, 6, 8, 3),
+    (10, 6, 4, 4, 3), (5, 1, 2, 3, 2), (4, 0, 4, 1, 1), (2, 3, 2, 5, 5), (8, 0, 1, 4, 1), (60, 4, 6, 8, 3),
     (300, 84, 32, 12, 5), (1, 1, 1, 2, 1), (6, 6, 4, 6, 4), (3, 0, 3, 3, 3)])
 def test_routing_by_corrected_scores_inside_the_best_groups(ops, experts, identity, top, count, keep):
     rng = np.random.default_rng(experts * 7 + identity)
@@ -369,7 +369,7 @@ def test_routing_among_equals_takes_the_lower_index_and_bars_groups_by_their_bes
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("width, experts, identity, top, ff, count, keep", [
     (64, 5, 1, 2, 24, 3, 2), (48, 3, 0, 1, 32, 1, 1), (512, 6, 2, 4, 520, 4, 3), (100, 4, 0, 4, 7, 2, 2),
-    (128, 8, 4, 4, 64, 4, 3), (192, 2, 6, 3, 96, 8, 5), (64, 1, 3, 4, 16, 2, 2),
+    (128, 8, 4, 4, 64, 4, 3), (160, 2, 6, 3, 80, 8, 5), (64, 1, 3, 4, 16, 2, 2),
     (128, 6, 2, 4, 4608, 4, 3)])  # the last: a token's hidden activations take more than 64 KB of LDS
 def test_mixture_with_identity_experts_against_the_plain_one(ops, dtype, width, experts, identity, top, ff, count, keep):
     from pylon_amd.config.specs import MixtureFeedForwardSpec
