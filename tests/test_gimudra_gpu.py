@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 F32_BOUND = 2e-4   # of a row's largest |logit|
 BF16_BOUND = 1e-1
-ROUTER_MARGIN = 0.004  # in bfloat16, choices between corrected scores (each below one) closer than this are accidents of rounding
+ROUTER_MARGIN = 0.008  # in bfloat16, choices between corrected scores (each below one) closer than this are accidents of rounding
 
 
 @pytest.fixture(scope="module")
@@ -468,7 +468,10 @@ class Case:
 
     def check(self, rid, got, label):
         clear = self.clear[rid][: len(got)]
-        assert clear.mean() >= 0.3, "too few positions with clear routing to compare"
+        assert clear.mean() >= getattr(self, "least_clear", 0.3), "too few positions with clear routing to compare"
+        assert np.isfinite(got).all()
+        if not clear.any():
+            return
         got, want = got[clear], self.want[rid][: len(got)][clear]
         ok, worst, frac = rows_within(got, want, self.bound if self.dtype == "float32" else 3 * self.bound)
         assert ok, f"{label}: request {rid}, position {np.flatnonzero(clear)[worst]} is off by {frac:.2e} of its largest logit"
@@ -647,3 +650,102 @@ def test_greedy_generation_through_the_engine(tmp, name, dtype, graphs, page):
             assert produced == int(row.argmax()) or row.max() - row[produced] <= slack * np.abs(row).max(), \
                 (prompt[:3], result.output_ids)
             sequence.append(produced)
+
+
+def draw_config(seed: int):
+    """A configuration drawn over what config.json allows: any order of layers with and without
+    keys and values of their own, heads and sizes in steps of 8 and a few odd ones, chunks that are no
+    multiple of anything, every shape of router."""
+    rng = np.random.default_rng(4000 + seed)
+    width = int(rng.choice([48, 64, 96, 136, 160, 256]))
+    layers, owners = [], []
+    for index in range(int(rng.integers(2, 7))):
+        borrow = owners and rng.random() < 0.45
+        if borrow:
+            lender = int(rng.choice(owners))
+            m = dict(layers[lender]["mixer"])
+            m.pop("kv_from", None)
+            m["kv_from"] = lender
+            m["scale"] = float(rng.uniform(0.05, 0.4))
+            if rng.random() < 0.3:
+                m["mask"] = {"size": int(rng.integers(3, 200))}
+        else:
+            kv_heads = int(rng.integers(1, 4))
+            dim = int(rng.choice([8, 16, 24, 32, 40, 64, 96, 128, 12]))
+            m = {"heads": kv_heads * int(rng.choice([1, 2, 3, 4, 8])), "kv_heads": kv_heads, "dim": dim,
+                 "vdim": int(rng.choice([4, 8, 20, 32, 48, 64, 80, 128, 10])), "scale": float(rng.uniform(0.05, 0.4)),
+                 "mask": {"size": int(rng.choice([int(rng.integers(3, 200)), 32, 64, 128, 1000]))}}
+            owners.append(index)
+        kind = rng.random()
+        if kind < 0.15:
+            mlp = None
+        elif kind < 0.4:
+            mlp = {"kind": "dense", "ff": 2 * int(rng.integers(8, 80))}
+        else:
+            count = int(rng.choice([1, 2, 3, 4, 6]))
+            per_group = int(rng.integers(1, 5))
+            outputs = count * per_group
+            identity = int(rng.integers(0, outputs))  # at least one expert
+            keep = int(rng.integers(1, count + 1))
+            top = int(rng.integers(1, min(keep * per_group, 8) + 1))
+            mlp = {"kind": "moe", "expert": {"ff": 8 * int(rng.integers(1, 12))},
+                   "router": {"experts": outputs - identity, "identity": identity, "top": top,
+                              "scale": float(rng.uniform(0.5, 3.0)), "groups": {"count": count, "keep": keep}}}
+        layers.append({"type": "attention", "mixer": m, "mlp": mlp})
+    config = {"architecture": "Gimudra", "vocab": int(rng.integers(90, 700)), "width": width,
+              "norm": {"eps": float(10 ** rng.uniform(-7, -4))}, "embedding": {"scale": float(rng.uniform(0.3, 3.0))},
+              "layers": layers}
+    return config, (int(rng.integers(1, 40)), int(rng.integers(60, 200)), int(rng.integers(200, 330)))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(10))
+def test_a_configuration_drawn_at_random_matches_the_plain_model(tmp, seed, dtype):
+    """Pages of 64 and four slots, as the replay program has them: each request whole, the longest with
+    its tail token by token, then all three side by side in portions over a pool too small for them
+    to have pages to spare."""
+    config, lengths = draw_config(seed)
+    case = Case.__new__(Case)
+    case.folder = make_folder(tmp, f"drawn{seed}", dtype=dtype, seed=seed, config=config)
+    case.cfg, case.weights = read_folder(case.folder)
+    case.requests = {f"r{i}": tokens(case.cfg["vocab"], n, 90 + i) for i, n in enumerate(lengths)}
+    case.want, case.clear = {}, {}
+    for rid, toks in case.requests.items():
+        margins = []
+        case.want[rid] = plain.forward(case.cfg, case.weights, toks, margins=margins)
+        closest = np.min(margins, axis=0) if margins else np.full(len(toks), np.inf)
+        if dtype == "float32":
+            case.clear[rid] = closest >= 1e-6
+        else:
+            # These routers are steep: bfloat16 rounding of their inputs moves scores by a hundredth, a
+            # flipped choice changes the token's whole feed-forward output, and the shift and the
+            # attention carry that to every later token.  Only the positions before the first
+            # unclear choice are held to the plain model; float32 holds them all.
+            unclear = np.flatnonzero(closest < 0.03)
+            case.clear[rid] = np.arange(len(toks)) < (unclear[0] if len(unclear) else len(toks))
+    case.dtype, case.bound = dtype, F32_BOUND if dtype == "float32" else BF16_BOUND
+    case.least_clear = 0.0
+    if sum(int(c.sum()) for c in case.clear.values()) < 40:
+        pytest.skip("too few positions with clear routing in this draw")
+    pages = sum(-(-n // 64) for n in lengths)
+    runner = case.runner(page_size=64, num_pages=pages, max_requests=4)
+    whole, _ = run_plan(runner, case, [{"r0": lengths[0]}, {"r0": 0, "r1": lengths[1]}, {"r1": 0, "r2": lengths[2]}])
+    for rid, got in whole.items():
+        case.check(rid, got, f"whole (seed {seed})")
+    tail, _ = run_plan(runner, case, [{"r2": lengths[2] - 70}] + [{"r2": 1}] * 70)
+    case.check("r2", tail["r2"], f"decoded tail (seed {seed})")
+    plan, left = [], dict(zip(("r0", "r1", "r2"), lengths))
+    sizes = iter(np.random.default_rng(seed).choice([1, 2, 3, 7, 31, 64, 65, 100], size=200).tolist())
+    while any(left.values()):
+        step = {}
+        for rid in left:
+            if left[rid]:
+                step[rid] = min(left[rid], next(sizes))
+                left[rid] -= step[rid]
+        plan.append(step)
+    mixed, _ = run_plan(runner, case, plan)
+    for rid, got in mixed.items():
+        case.check(rid, got, f"portions side by side (seed {seed})")
+        if dtype == "float32":
+            assert np.abs(got - whole[rid]).max() <= 2e-5 * np.abs(whole[rid]).max(), (seed, rid)
+    assert runner.manager.free_pages == pages
