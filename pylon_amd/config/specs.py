@@ -27,12 +27,28 @@ class NormSpec:
 
 
 @dataclass(frozen=True)
+class RotaryScalingSpec:
+    """Frequencies stretched for contexts longer than the ``original`` one: with ``where(t) =
+    rotary_dim * ln(original / (2 pi t)) / (2 ln theta)`` the (fractional) pair that makes ``t`` turns
+    over the original length, ``lo = max(floor(where(fast)), 0)``, ``hi = min(ceil(where(slow)),
+    rotary_dim - 1)`` and ``ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)``, pair ``i`` turns
+    at ``f_i / factor * ramp_i + f_i * (1 - ramp_i)``, and every cosine and sine is multiplied by
+    ``0.1 * ln(factor) + 1``."""
+
+    factor: float
+    original: float
+    fast: float
+    slow: float
+
+
+@dataclass(frozen=True)
 class PositionSpec:
     """How positions enter a mixer.
 
     ``kind="rope"``: rotate the first ``rotary_dim`` elements of every head by
     ``position * theta**(-2i/rotary_dim)``, pairing element ``i`` with
     ``i + rotary_dim/2``.  ``kind="none"``: positions are not encoded.
+    ``scaling``: see :class:`RotaryScalingSpec`.
     """
 
     kind: str
@@ -41,6 +57,7 @@ class PositionSpec:
     max_positions: int = 0
     # True: element 2i turns together with its neighbour 2i + 1 instead of with i + rotary_dim/2
     interleaved: bool = False
+    scaling: Optional[RotaryScalingSpec] = None
 
 
 @dataclass(frozen=True)
@@ -64,10 +81,29 @@ class AttentionSpec:
     # c: position i sees key j <= i only if floor(i / c) == floor(j / c), chunks counted from the
     # request's first token (not together with a window)
     chunk: Optional[int] = None
+    # the scaled score s becomes softcap * tanh(s / softcap)
+    softcap: Optional[float] = None
+    # True: a learned number per head joins the softmax's denominator as exp(sink_h): a key without
+    # a value whose score is neither scaled nor capped
+    sink: bool = False
+    # "head": every head's output is multiplied by sigmoid(W_g h) of that head (W_g has one row a
+    # head); "element": the concatenated heads element by element (one row an element); both read
+    # the mixer's input, as the projections do
+    output_gate: Optional[str] = None
+    # True: there is no value projection; the values are the keys as projected, before their norm
+    # and rotation
+    values_from_keys: bool = False
 
     @property
     def q_size(self) -> int:
         return self.n_heads * self.head_dim
+
+    @property
+    def gate_size(self) -> int:
+        """Rows of the gate's projection."""
+        if self.output_gate is None:
+            return 0
+        return self.n_heads if self.output_gate == "head" else self.n_heads * self.value_dim
 
     @property
     def kv_size(self) -> int:
@@ -162,6 +198,40 @@ class RetentionSpec:
 
 
 @dataclass(frozen=True)
+class DeltaRuleSpec:
+    """The gated delta rule: per request and head a float32 state ``S`` of ``head_dim x v_head_dim``,
+    ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q`` (the read-out sees the token's own
+    write).  ``q`` and ``k`` have ``n_kv_heads`` heads (head ``h`` uses ``h // (n_heads / n_kv_heads)``),
+    ``v`` has ``n_heads``; each of the three passes a causal convolution of ``conv_taps`` taps per
+    channel and ``silu``; q and k become unit vectors per head (``unit_eps`` inside the root), q also
+    times ``head_dim ** -0.5``; ``beta = sigmoid(W_b h)``, ``g = exp(-exp(A_log) * softplus(W_a h +
+    dt_bias))`` per head; every head's ``o`` is divided by its root mean square (``norm_eps``), times a
+    weight shared by the heads, times ``silu(W_g h)``; then the output projection."""
+
+    hidden_size: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    v_head_dim: int
+    conv_taps: int
+    norm_eps: float
+    unit_eps: float = 1e-6
+    kind: str = "delta_rule"
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """Two mixers side by side on the same input: ``left_scale * left(h) + right_scale * right(h)``;
+    ``left`` and ``right`` are mixer specs of any kind (at most one of them keeps keys and values)."""
+
+    left: object
+    right: object
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    kind: str = "parallel"
+
+
+@dataclass(frozen=True)
 class TokenShiftSpec:
     """``h + (h' - h) * w``: every token's input moved towards the previous token's (``h'``, zeros
     before a request's first token) by a learned share per channel; a request's last input is its
@@ -218,7 +288,11 @@ class MixtureFeedForwardSpec:
     which only the ``groups_kept`` with the largest corrected score can be chosen from; the weights
     are the chosen scores times ``route_scale``, not renormalised.  The router's last ``n_identity``
     outputs (beyond the ``n_experts`` experts, and counted in the groups) are identity experts whose
-    output is the input itself."""
+    output is the input itself.
+
+    ``scoring="sigmoid"``: the scores are the sigmoids of the router's outputs, the ``top`` largest
+    are chosen and their scores are the weights as they are.  ``weight_on_input``: a chosen expert's
+    weight multiplies its input instead of its output, ``sum_e expert_e(w_e h)``."""
 
     hidden_size: int
     n_experts: int
@@ -234,6 +308,7 @@ class MixtureFeedForwardSpec:
     groups: int = 1
     groups_kept: int = 1
     route_scale: float = 1.0
+    weight_on_input: bool = False
 
 
 @dataclass(frozen=True)

@@ -10,7 +10,9 @@
 // rel[bucket[min(i - j, bucket_len - 1)] * n_heads + head], or without a table of buckets a bias
 // that grows with the logarithm of the distance and is taken off, rel[head] * log(1 + rel[n_heads +
 // head] * (i - j)); and a sink, a key of score 0 without a value, which adds one to the softmax's
-// denominator.
+// denominator, or with sink_logit a learned score per head in its place (exp(sink_logit[head]) is
+// added; it is neither scaled nor capped).  softcap > 0: the scaled score s becomes softcap *
+// tanh(s / softcap) before anything is added to it.
 #include "common.h"
 
 #define ATT_WAVES 4
@@ -57,7 +59,8 @@ __global__ void paged_attention_kernel(T* __restrict__ out, const T* __restrict_
                                        long long items, int n_heads, int n_kv_heads, int head_dim,
                                        int page_size, int window, float scale, int v_dim, long long q_stride,
                                        const float* __restrict__ rel, const int* __restrict__ bucket,
-                                       int bucket_len, int sink, int v_transposed) {
+                                       int bucket_len, int sink, int v_transposed, float softcap,
+                                       const float* __restrict__ sink_logit) {
   extern __shared__ float lds[];
   const int lane = threadIdx.x & (PYLON_WAVE - 1);
   const int wave = threadIdx.x / PYLON_WAVE;
@@ -99,6 +102,7 @@ __global__ void paged_attention_kernel(T* __restrict__ out, const T* __restrict_
         for (int d = 0; d < head_dim; d += 8) dot = Vec8<T>::dot(qbuf + d, kr + d, dot);
       }
       s = dot * scale;
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
       if (rel != nullptr) {
         const int far = pos - j;
         if (bucket != nullptr)
@@ -132,7 +136,17 @@ __global__ void paged_attention_kernel(T* __restrict__ out, const T* __restrict_
     m = m_new;
   }
   T* orow = out + (static_cast<size_t>(t) * n_heads + h) * v_dim;
-  if (sink) l += expf(-m);  // the sink's weight on the scale of the running maximum
+  if (sink_logit != nullptr) {
+    // the sink joins as one more score: the larger of it and the maximum so far is the new scale
+    const float z = sink_logit[h];
+    const float m_fin = fmaxf(m, z);
+    const float corr = expf(m - m_fin);
+    l = l * corr + expf(z - m_fin);
+#pragma unroll
+    for (int i = 0; i < DIMS_PER_LANE; ++i) acc[i] *= corr;
+  } else if (sink) {
+    l += expf(-m);  // the sink's weight on the scale of the running maximum
+  }
   const float inv = 1.0f / l;
 #pragma unroll
   for (int i = 0; i < DIMS_PER_LANE; ++i) {
@@ -147,7 +161,8 @@ static int launch_paged_attention(T* out, const T* q, const T* k_cache, const T*
                                   const int* positions, int tokens, int n_heads, int n_kv_heads,
                                   int head_dim, int page_size, int window, float scale, int v_dim,
                                   long long q_stride, const float* rel, const int* bucket, int bucket_len,
-                                  int sink, int v_transposed, hipStream_t stream) {
+                                  int sink, int v_transposed, float softcap, const float* sink_logit,
+                                  hipStream_t stream) {
   const long long items = static_cast<long long>(tokens) * n_heads;
   const long long blocks = (items + ATT_WAVES - 1) / ATT_WAVES;
   dim3 grid((unsigned)blocks), block(ATT_WAVES * PYLON_WAVE);
@@ -156,7 +171,7 @@ static int launch_paged_attention(T* out, const T* q, const T* k_cache, const T*
   hipLaunchKernelGGL((paged_attention_kernel<T, DPL>), grid, block, lds, stream, out, q, k_cache,    \
                      v_cache, block_table, table_width, tok_row, positions, items, n_heads,          \
                      n_kv_heads, head_dim, page_size, window, scale, v_dim, q_stride, rel, bucket,   \
-                     bucket_len, sink, v_transposed)
+                     bucket_len, sink, v_transposed, softcap, sink_logit)
   if (v_dim <= 64)
     LAUNCH(1);
   else if (v_dim <= 128)
@@ -184,7 +199,7 @@ extern "C" int pylon_paged_attention(void* out, const void* q, const void* k_cac
                                      int n_kv_heads, int head_dim, int page_size, int window,
                                      float scale, int v_dim, long long q_stride, const float* rel,
                                      const int* bucket, int bucket_len, int sink, int v_transposed,
-                                     hipStream_t stream) {
+                                     float softcap, const float* sink_logit, hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(dtype), "paged_attention: unknown dtype");
   PYLON_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                 "paged_attention: %d query heads cannot be grouped over %d key/value heads", n_heads,
@@ -202,11 +217,13 @@ extern "C" int pylon_paged_attention(void* out, const void* q, const void* k_cac
     launch_paged_attention<float>((float*)out, (const float*)q, (const float*)k_cache,
                                   (const float*)v_cache, block_table, table_width, tok_row, positions,
                                   tokens, n_heads, n_kv_heads, head_dim, page_size, window, scale, v_dim,
-                                  q_stride, rel, bucket, bucket_len, sink, v_transposed, stream);
+                                  q_stride, rel, bucket, bucket_len, sink, v_transposed, softcap, sink_logit,
+                                  stream);
   else
     launch_paged_attention<bf16_t>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache,
                                    (const bf16_t*)v_cache, block_table, table_width, tok_row, positions,
                                    tokens, n_heads, n_kv_heads, head_dim, page_size, window, scale, v_dim,
-                                   q_stride, rel, bucket, bucket_len, sink, v_transposed, stream);
+                                   q_stride, rel, bucket, bucket_len, sink, v_transposed, softcap, sink_logit,
+                                  stream);
   PYLON_LAUNCHED("paged_attention");
 }

@@ -583,3 +583,73 @@ extern "C" int pylon_add_bias(void* x, int dtype, const float* bias, long long r
     hipLaunchKernelGGL(add_bias_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, (bf16_t*)x, bias, dim, total);
   PYLON_LAUNCHED("add_bias");
 }
+
+// ---- a sigmoid gate on a mixer's heads, in place ---------------------------------------------------
+// x[t, i] *= sigmoid(g[t, i / per]): per = the size of a head for one gate per head, 1 for a gate
+// per element.  The gates' logits lie in rows g_stride apart (a slice of a wider projection).
+template <typename T>
+__global__ void sigmoid_gate_kernel(T* __restrict__ x, const T* __restrict__ g, long long g_stride, int dim, int per,
+                                    size_t total) {
+  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (; i < total; i += step) {
+    const size_t t = i / dim;
+    const int e = static_cast<int>(i - t * dim);
+    const float z = to_float(g[t * g_stride + e / per]);
+    x[i] = from_float<T>(to_float(x[i]) / (1.0f + expf(-z)));
+  }
+}
+
+// x: [rows, dim] of dtype, contiguous; g: [rows, dim / per] of the same dtype, rows g_stride apart.
+extern "C" int pylon_sigmoid_gate(void* x, int dtype, const void* g, long long g_stride, long long rows, int dim,
+                                  int per, hipStream_t stream) {
+  PYLON_REQUIRE(pylon_valid_dtype(dtype) && rows >= 0 && dim > 0 && per > 0 && dim % per == 0,
+                "sigmoid_gate: bad arguments");
+  PYLON_REQUIRE(g_stride >= dim / per, "sigmoid_gate: rows of gates overlap");
+  const size_t total = static_cast<size_t>(rows) * dim;
+  if (total == 0) return 0;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65535u * 16u) blocks = 65535u * 16u;
+  if (dtype == PYLON_F32)
+    hipLaunchKernelGGL(sigmoid_gate_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, (float*)x,
+                       (const float*)g, g_stride, dim, per, total);
+  else
+    hipLaunchKernelGGL(sigmoid_gate_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, (bf16_t*)x,
+                       (const bf16_t*)g, g_stride, dim, per, total);
+  PYLON_LAUNCHED("sigmoid_gate");
+}
+
+// ---- two mixers side by side: out = sa * a + sb * b, float ----------------------------------------
+// a and b are each one tensor of n elements, or a stack of float partial sums that are added up in
+// order first (parts > 1: the parts lie n elements apart).
+template <typename TA, typename TB>
+__global__ void scaled_sum_kernel(float* __restrict__ out, const TA* __restrict__ a, int a_parts, float sa,
+                                  const TB* __restrict__ b, int b_parts, float sb, size_t n) {
+  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (; i < n; i += step) {
+    float x = to_float(a[i]);
+    for (int p = 1; p < a_parts; ++p) x += to_float(a[i + p * n]);
+    float y = to_float(b[i]);
+    for (int p = 1; p < b_parts; ++p) y += to_float(b[i + p * n]);
+    out[i] = fmaf(sa, x, sb * y);
+  }
+}
+
+extern "C" int pylon_scaled_sum(float* out, const void* a, int a_dtype, int a_parts, float sa, const void* b,
+                                int b_dtype, int b_parts, float sb, long long n, hipStream_t stream) {
+  PYLON_REQUIRE(pylon_valid_dtype(a_dtype) && pylon_valid_dtype(b_dtype) && n >= 0 && a_parts >= 1 && b_parts >= 1,
+                "scaled_sum: bad arguments");
+  if (n == 0) return 0;
+  size_t blocks = (static_cast<size_t>(n) + 255) / 256;
+  if (blocks > 65535u * 16u) blocks = 65535u * 16u;
+#define GO(TA, TB)                                                                                          \
+  hipLaunchKernelGGL((scaled_sum_kernel<TA, TB>), dim3((unsigned)blocks), dim3(256), 0, stream, out,        \
+                     (const TA*)a, a_parts, sa, (const TB*)b, b_parts, sb, static_cast<size_t>(n))
+  if (a_dtype == PYLON_F32 && b_dtype == PYLON_F32) GO(float, float);
+  else if (a_dtype == PYLON_F32) GO(float, bf16_t);
+  else if (b_dtype == PYLON_F32) GO(bf16_t, float);
+  else GO(bf16_t, bf16_t);
+#undef GO
+  PYLON_LAUNCHED("scaled_sum");
+}

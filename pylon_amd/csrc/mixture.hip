@@ -2,8 +2,9 @@
 //
 // route_top: from float router logits (a product computed elsewhere) plus a bias, the `top`
 //   experts with the largest logits (the lower index among equals) and the softmax over those
-//   logits alone; optionally sigmoid of one more logit per token, the gate of a shared expert.
-//   One wavefront per token, everything in float.
+//   logits alone (scoring 0), or every chosen expert's own sigmoid(logit) as it is (scoring 1: the
+//   order of the sigmoids is the order of the logits); optionally sigmoid of one more logit per
+//   token, the gate of a shared expert.  One wavefront per token, everything in float.
 // expert_gate_up: hidden[(t, s)] = silu(W_gate[e] x_t) * (W_up[e] x_t) for every token t and each of
 //   its chosen experts e = experts[t, s]; a workgroup takes one (token, choice) and some hidden
 //   units, the token's input in LDS, a wave a hidden unit at a time with the lanes along the row.
@@ -24,7 +25,7 @@
 __global__ void __launch_bounds__(256)
 route_top_kernel(int* __restrict__ experts, float* __restrict__ weights, float* __restrict__ shared_gate,
                  const float* __restrict__ logits, long long row_stride, const float* __restrict__ bias,
-                 int tokens, int n_experts, int top) {
+                 int tokens, int n_experts, int top, int scoring) {
   __shared__ float chosen[4][MX_MAX_TOP];
   const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
   const int t = blockIdx.x * 4 + wave;
@@ -69,14 +70,19 @@ route_top_kernel(int* __restrict__ experts, float* __restrict__ weights, float* 
   }
   __builtin_amdgcn_wave_barrier();
   if (lane == 0) {
-    const float m = chosen[wave][0];  // the largest: they were taken in falling order
-    float sum = 0.f;
-    for (int k = 0; k < top; ++k) {
-      const float p = expf(chosen[wave][k] - m);
-      chosen[wave][k] = p;
-      sum += p;
+    if (scoring == 1) {
+      for (int k = 0; k < top; ++k)
+        weights[static_cast<size_t>(t) * top + k] = 1.0f / (1.0f + expf(-chosen[wave][k]));
+    } else {
+      const float m = chosen[wave][0];  // the largest: they were taken in falling order
+      float sum = 0.f;
+      for (int k = 0; k < top; ++k) {
+        const float p = expf(chosen[wave][k] - m);
+        chosen[wave][k] = p;
+        sum += p;
+      }
+      for (int k = 0; k < top; ++k) weights[static_cast<size_t>(t) * top + k] = chosen[wave][k] / sum;
     }
-    for (int k = 0; k < top; ++k) weights[static_cast<size_t>(t) * top + k] = chosen[wave][k] / sum;
     if (shared_gate != nullptr) shared_gate[t] = 1.0f / (1.0f + expf(-row[n_experts]));
   }
 }
@@ -85,7 +91,8 @@ route_top_kernel(int* __restrict__ experts, float* __restrict__ weights, float* 
 // float [n_experts]; experts int [tokens, top], weights float [tokens, top], shared_gate null or float [tokens].
 extern "C" int pylon_route_top(int* experts, float* weights, float* shared_gate, const float* logits,
                                long long row_stride, const float* bias, int tokens, int n_experts, int top,
-                               hipStream_t stream) {
+                               int scoring, hipStream_t stream) {
+  PYLON_REQUIRE(scoring == 0 || scoring == 1, "route_top: unknown scoring %d", scoring);
   PYLON_REQUIRE(tokens >= 0 && n_experts >= 1 && n_experts <= 8 * PYLON_WAVE,
                 "route_top: 1 to %d experts, got %d", 8 * PYLON_WAVE, n_experts);
   PYLON_REQUIRE(top >= 1 && top <= n_experts && top <= MX_MAX_TOP, "route_top: top %d of %d experts (at most %d)",
@@ -93,7 +100,7 @@ extern "C" int pylon_route_top(int* experts, float* weights, float* shared_gate,
   PYLON_REQUIRE(row_stride >= n_experts + (shared_gate != nullptr ? 1 : 0), "route_top: rows of logits overlap");
   if (tokens == 0) return 0;
   hipLaunchKernelGGL(route_top_kernel, dim3((tokens + 3) / 4), dim3(256), 0, stream, experts, weights, shared_gate,
-                     logits, row_stride, bias, tokens, n_experts, top);
+                     logits, row_stride, bias, tokens, n_experts, top, scoring);
   PYLON_LAUNCHED("route_top");
 }
 
@@ -367,13 +374,16 @@ template <typename TX, typename TW>
 __global__ void __launch_bounds__(256)
 expert_gate_up_kernel(TX* __restrict__ hidden, const TX* __restrict__ x, long long x_stride,
                       const TW* __restrict__ w, long long w_stride, const int* __restrict__ experts, int top,
-                      int ff, int width, int units_per_block, int wide, int act, int n_experts) {
+                      int ff, int width, int units_per_block, int wide, int act, int n_experts,
+                      const float* __restrict__ in_weights) {
   extern __shared__ float xs[];  // the token's input
   const int pair = blockIdx.y, t = pair / top;
   const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
   const int e = experts[pair];
   if (e >= n_experts) return;  // an identity: nothing to compute (the whole workgroup, before any barrier)
-  for (int i = threadIdx.x; i < width; i += 256) xs[i] = to_float(x[static_cast<size_t>(t) * x_stride + i]);
+  // with in_weights the expert works on the token's input times the pair's weight (float in LDS)
+  const float in_w = in_weights != nullptr ? in_weights[pair] : 1.f;
+  for (int i = threadIdx.x; i < width; i += 256) xs[i] = to_float(x[static_cast<size_t>(t) * x_stride + i]) * in_w;
   __syncthreads();
   const int j0 = blockIdx.x * units_per_block;
   const int j1 = j0 + units_per_block < ff ? j0 + units_per_block : ff;
@@ -442,9 +452,11 @@ expert_gate_up_kernel(TX* __restrict__ hidden, const TX* __restrict__ x, long lo
 // expert's gate rows then its up rows; experts: int [tokens, top]; hidden: [tokens * top, ff].
 // act 1: plain experts, w [n_experts, ff, width], hidden = relu(W_up x)^2.  A pair whose expert is
 // n_experts or more (an identity) is passed over: its rows of hidden stay as they are.
+// in_weights: null, or float [tokens, top]: a pair's expert works on x times the pair's weight.
 extern "C" int pylon_expert_gate_up(void* hidden, const void* x, int x_dtype, long long x_stride, const void* w,
                                     int w_dtype, long long w_stride, const int* experts, int tokens, int top, int ff,
-                                    int width, int act, int n_experts, hipStream_t stream) {
+                                    int width, int act, int n_experts, const float* in_weights,
+                                    hipStream_t stream) {
   PYLON_REQUIRE(act == 0 || act == 1, "expert_gate_up: unknown activation %d", act);
   PYLON_REQUIRE(pylon_valid_dtype(x_dtype) && pylon_valid_dtype(w_dtype), "expert_gate_up: unknown dtype");
   PYLON_REQUIRE(!(x_dtype == PYLON_F32 && w_dtype == PYLON_BF16), "expert_gate_up: float inputs take float weights");
@@ -467,7 +479,7 @@ extern "C" int pylon_expert_gate_up(void* hidden, const void* x, int x_dtype, lo
 #define GO(TX, TW)                                                                                               \
   hipLaunchKernelGGL((expert_gate_up_kernel<TX, TW>), grid, block, lds, stream, (TX*)hidden + off * ff,          \
                      (const TX*)x + (off / top) * x_stride, x_stride, (const TW*)w, w_stride, experts + off, top, \
-                     ff, width, units, wide, act, n_experts)
+                     ff, width, units, wide, act, n_experts, in_weights != nullptr ? in_weights + off : nullptr)
     if (x_dtype == PYLON_F32) GO(float, float);
     else if (w_dtype == PYLON_F32) GO(bf16_t, float);
     else GO(bf16_t, bf16_t);
@@ -636,7 +648,8 @@ template <int ACT, int MT, typename TO>
 __global__ void __launch_bounds__(256)
 grouped_rows_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restrict__ x, long long ldx,
                     const int* __restrict__ row_index, const uint16_t* __restrict__ w, long long ldw,
-                    long long expert_rows, const int* __restrict__ offsets, int n_experts, int N, int K) {
+                    long long expert_rows, const int* __restrict__ offsets, int n_experts, int N, int K,
+                    const float* __restrict__ row_scale) {
   constexpr bool GLU = ACT == 1;  // ACT: 0 the sums as they are, 1 silu(gate) * up, 2 the square of relu
   constexpr int MX_TM = 16 * MT;  // rows of a tile
   constexpr int J = GLU ? 4 : 2;  // weight tiles of a wave: GLU: two of gate rows, then the two of their up rows
@@ -708,14 +721,16 @@ grouped_rows_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restr
   for (int t = 0; t < MT; ++t) {
     if (16 * t + r >= rows) continue;
     TO* orow = out + static_cast<size_t>(row0 + 16 * t + r) * ldo;
+    // a row's scale: the products are linear, so the sums of the scaled input are the scaled sums
+    const float rs = row_scale != nullptr ? row_scale[row0 + 16 * t + r] : 1.f;
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int n = n0 + 16 * j + 4 * g + i;
         if (n >= N) continue;
-        float v = acc[j][t][i];
-        if constexpr (GLU) v = v / (1.0f + expf(-v)) * acc[2 + j][t][i];
+        float v = acc[j][t][i] * rs;
+        if constexpr (GLU) v = v / (1.0f + expf(-v)) * (acc[2 + j][t][i] * rs);
         if constexpr (ACT == 2) v = fmaxf(v, 0.f) * fmaxf(v, 0.f);
         orow[n] = from_float<TO>(v);
       }
@@ -738,7 +753,8 @@ template <int ACT, typename TO>
 __global__ void __launch_bounds__(256, 2)
 grouped_tiles_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restrict__ x, long long ldx,
                      const int* __restrict__ row_index, const uint16_t* __restrict__ w, long long ldw,
-                     long long expert_rows, const int* __restrict__ offsets, int n_experts, int N, int K) {
+                     long long expert_rows, const int* __restrict__ offsets, int n_experts, int N, int K,
+                     const float* __restrict__ row_scale) {
   constexpr bool GLU = ACT == 1;
   constexpr int WROWS = 2 * GT_COLS;  // GLU: 128 gate rows and their 128 up rows; else 256 output columns
   constexpr int TILE_COLS = GLU ? GT_COLS : 2 * GT_COLS, WAVE_COLS = TILE_COLS / 4;
@@ -822,14 +838,15 @@ grouped_tiles_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __rest
   for (int t = 0; t < MT; ++t) {
     if (16 * t + r >= rows) continue;
     TO* orow = out + static_cast<size_t>(row0 + 16 * t + r) * ldo;
+    const float rs = row_scale != nullptr ? row_scale[row0 + 16 * t + r] : 1.f;
 #pragma unroll
     for (int j = 0; j < (GLU ? 2 : J); ++j)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int n = n0 + WAVE_COLS * wave + 16 * j + 4 * g + i;
         if (n >= N) continue;
-        float v = acc[j][t][i];
-        if constexpr (GLU) v = v / (1.0f + expf(-v)) * acc[2 + j][t][i];
+        float v = acc[j][t][i] * rs;
+        if constexpr (GLU) v = v / (1.0f + expf(-v)) * (acc[2 + j][t][i] * rs);
         if constexpr (ACT == 2) v = fmaxf(v, 0.f) * fmaxf(v, 0.f);
         orow[n] = from_float<TO>(v);
       }
@@ -857,10 +874,12 @@ static int grouped_checks(const char* name, const void* x, long long ldx, const 
 // every expert e (offsets: int [n_experts + 1]); x bfloat16 [tokens, width]; w bfloat16
 // [n_experts * 2 ff, width]; hidden bfloat16 [pairs, ff]; tokens_bound: the rows of x.  act 1: plain
 // experts, hidden[p] = relu(W_up[e] x)^2 with w [n_experts * ff, width].  pairs counts the sorted
-// pairs of these n_experts experts only (identities' pairs lie behind them).
+// pairs of these n_experts experts only (identities' pairs lie behind them).  row_scale: null, or
+// float [pairs]: sorted pair p's expert works on its input times row_scale[p] (gated experts).
 extern "C" int pylon_grouped_gate_up(void* hidden, const void* x, long long ldx, const int* row_index, const void* w,
                                      long long ldw, const int* offsets, int pairs, int n_experts, int ff, int width,
-                                     int tokens_bound, int act, hipStream_t stream) {
+                                     int tokens_bound, int act, const float* row_scale, hipStream_t stream) {
+  PYLON_REQUIRE(row_scale == nullptr || act == 0, "grouped_gate_up: a scale per pair goes with gated experts");
   if (grouped_checks("grouped_gate_up", x, ldx, w, ldw, width, ff, pairs, n_experts)) return 1;
   PYLON_REQUIRE(act == 0 || act == 1, "grouped_gate_up: unknown activation %d", act);
   if (pairs == 0) return 0;
@@ -873,11 +892,11 @@ extern "C" int pylon_grouped_gate_up(void* hidden, const void* x, long long ldx,
     if (large1)
       hipLaunchKernelGGL((grouped_tiles_kernel<2, bf16_t>), grid1, block1, 0, stream, (bf16_t*)hidden, (long long)ff,
                          (const uint16_t*)x, ldx, row_index, (const uint16_t*)w, ldw, (long long)ff, offsets, n_experts,
-                         ff, width);
+                         ff, width, nullptr);
     else
       hipLaunchKernelGGL((grouped_rows_kernel<2, 4, bf16_t>), grid1, block1, 0, stream, (bf16_t*)hidden, (long long)ff,
                          (const uint16_t*)x, ldx, row_index, (const uint16_t*)w, ldw, (long long)ff, offsets, n_experts,
-                         ff, width);
+                         ff, width, nullptr);
     PYLON_LAUNCHED("grouped_gate_up");
   }
   const bool large = grouped_large(pairs, n_experts, tokens_bound * ldx, 2ll * n_experts * ff * ldw);
@@ -887,11 +906,11 @@ extern "C" int pylon_grouped_gate_up(void* hidden, const void* x, long long ldx,
   if (large)
     hipLaunchKernelGGL((grouped_tiles_kernel<1, bf16_t>), grid, block, 0, stream, (bf16_t*)hidden, (long long)ff,
                        (const uint16_t*)x, ldx, row_index, (const uint16_t*)w, ldw, 2ll * ff, offsets, n_experts, ff,
-                       width);
+                       width, row_scale);
   else
     hipLaunchKernelGGL((grouped_rows_kernel<1, 4, bf16_t>), grid, block, 0, stream, (bf16_t*)hidden,
                        (long long)ff, (const uint16_t*)x, ldx, row_index, (const uint16_t*)w, ldw, 2ll * ff, offsets,
-                       n_experts, ff, width);
+                       n_experts, ff, width, row_scale);
   PYLON_LAUNCHED("grouped_gate_up");
 }
 
@@ -909,11 +928,11 @@ extern "C" int pylon_grouped_down(float* y, const void* hidden, long long ldh, c
   if (large)
     hipLaunchKernelGGL((grouped_tiles_kernel<0, float>), grid, block, 0, stream, y, (long long)width,
                        (const uint16_t*)hidden, ldh, nullptr, (const uint16_t*)w, ldw, (long long)width, offsets,
-                       n_experts, width, ff);
+                       n_experts, width, ff, nullptr);
   else
     hipLaunchKernelGGL((grouped_rows_kernel<0, 4, float>), grid, block, 0, stream, y, (long long)width,
                        (const uint16_t*)hidden, ldh, nullptr, (const uint16_t*)w, ldw, (long long)width, offsets,
-                       n_experts, width, ff);
+                       n_experts, width, ff, nullptr);
   PYLON_LAUNCHED("grouped_down");
 }
 

@@ -2,7 +2,9 @@
 //
 //   out[t, c] = h[t, c] + sum_{j < taps} w[c, j] * h[t - taps + 1 + j, c]
 //
-// with zeros before a request's first token.  The last taps - 1 inputs of every request are
+// with zeros before a request's first token; or, with mode 1, the convolution alone through an
+// activation, out[t, c] = silu(sum_j w[c, j] * h[t - taps + 1 + j, c]).  The rows of h may lie
+// further apart than width (a slice of a wider projection).  The last taps - 1 inputs of every request are
 // kept in its state slot, float [taps - 1, width] (oldest first), so that a request may come
 // in portions: a portion's first tokens read what the portion before left there.
 //
@@ -18,7 +20,8 @@
 template <typename TI, typename TW, typename TO>
 __global__ void short_conv_kernel(TO* __restrict__ out, const TI* __restrict__ h, const TW* __restrict__ w,
                                   float* state, const int* __restrict__ row_start,
-                                  const int* __restrict__ row_slots, int tiles_per_row, int width, int taps) {
+                                  const int* __restrict__ row_slots, int tiles_per_row, int width, int taps,
+                                  long long h_stride, int mode) {
   const int row = blockIdx.x / tiles_per_row;
   const int tile = blockIdx.x - row * tiles_per_row;
   const int begin = row_start[row], end = row_start[row + 1];
@@ -47,14 +50,14 @@ __global__ void short_conv_kernel(TO* __restrict__ out, const TI* __restrict__ h
   for (int j = 0; j < CONV_MAX_TAPS - 1; ++j) {
     if (j < keep) {
       const int src = a - keep + j;  // token index of the step
-      if (src >= begin) win[j + 1] = to_float(h[static_cast<size_t>(src) * width + c]);
+      if (src >= begin) win[j + 1] = to_float(h[static_cast<size_t>(src) * h_stride + c]);
       else if (first_tile) win[j + 1] = old[keep - (begin - src)];
     }
   }
   // a tile's inputs are fetched before the first sum, so that their trips to memory overlap
   float xs[CONV_TILE];
 #pragma unroll
-  for (int n = 0; n < CONV_TILE; ++n) xs[n] = (a + n < b) ? to_float(h[static_cast<size_t>(a + n) * width + c]) : 0.f;
+  for (int n = 0; n < CONV_TILE; ++n) xs[n] = (a + n < b) ? to_float(h[static_cast<size_t>(a + n) * h_stride + c]) : 0.f;
 #pragma unroll
   for (int n = 0; n < CONV_TILE; ++n) {
     const int t = a + n;
@@ -69,7 +72,7 @@ __global__ void short_conv_kernel(TO* __restrict__ out, const TI* __restrict__ h
 #pragma unroll
     for (int j = 0; j < CONV_MAX_TAPS; ++j)
       if (j < taps) acc = fmaf(wt[j], win[j], acc);
-    out[static_cast<size_t>(t) * width + c] = from_float<TO>(x + acc);
+    out[static_cast<size_t>(t) * width + c] = from_float<TO>(mode == 1 ? acc / (1.0f + expf(-acc)) : x + acc);
   }
   if (first_tile) {
 #pragma unroll
@@ -77,7 +80,7 @@ __global__ void short_conv_kernel(TO* __restrict__ out, const TI* __restrict__ h
       if (i < keep) {
         const int src = end - keep + i;
         float v;
-        if (src >= begin) v = to_float(h[static_cast<size_t>(src) * width + c]);
+        if (src >= begin) v = to_float(h[static_cast<size_t>(src) * h_stride + c]);
         else v = old[keep - (begin - src)];
         st[static_cast<size_t>(i) * width] = v;
       }
@@ -85,18 +88,20 @@ __global__ void short_conv_kernel(TO* __restrict__ out, const TI* __restrict__ h
   }
 }
 
-// h: [tokens, width] of in_dtype; w: [width, taps] of w_dtype; out: [tokens, width] of out_dtype;
+// h: [tokens, width] of in_dtype, rows h_stride elements apart; w: [width, taps] of w_dtype; out:
+// [tokens, width] of out_dtype; mode 0: input plus convolution, 1: silu of the convolution;
 // state: float [slots, taps - 1, width]; row_start: [rows + 1] prefix sums of the rows' token
 // counts; row_slots: [rows] state slot of each row; max_count: the most tokens any row brings
 // (an upper bound will do).  The host guarantees row_slots < slots and row_start[rows] <= tokens.
 extern "C" int pylon_short_conv(void* out, int out_dtype, const void* h, int in_dtype, const void* w, int w_dtype,
                                 float* state, const int* row_start, const int* row_slots, int rows, int max_count,
-                                int width, int taps, hipStream_t stream) {
+                                int width, int taps, long long h_stride, int mode, hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(out_dtype) && pylon_valid_dtype(in_dtype) && pylon_valid_dtype(w_dtype),
                 "short_conv: unknown dtype");
   PYLON_REQUIRE(taps >= 1 && taps <= CONV_MAX_TAPS, "short_conv: 1 to %d taps, got %d", CONV_MAX_TAPS, taps);
   PYLON_REQUIRE(CONV_TILE >= CONV_MAX_TAPS, "short_conv: a tile must hold a window");
   PYLON_REQUIRE(rows >= 0 && max_count >= 0 && width > 0, "short_conv: bad sizes");
+  PYLON_REQUIRE(h_stride >= width && (mode == 0 || mode == 1), "short_conv: rows overlap, or an unknown mode");
   PYLON_REQUIRE(taps == 1 || state != nullptr, "short_conv: a window over several tokens needs its state");
   if (rows == 0 || max_count == 0) return 0;
   const int tiles_per_row = (max_count + CONV_TILE - 1) / CONV_TILE;
@@ -104,7 +109,7 @@ extern "C" int pylon_short_conv(void* out, int out_dtype, const void* h, int in_
   dim3 grid(static_cast<unsigned>(rows * tiles_per_row), (width + 255) / 256), block(256);
 #define GO(TI, TW, TO)                                                                                       \
   hipLaunchKernelGGL((short_conv_kernel<TI, TW, TO>), grid, block, 0, stream, (TO*)out, (const TI*)h,        \
-                     (const TW*)w, state, row_start, row_slots, tiles_per_row, width, taps)
+                     (const TW*)w, state, row_start, row_slots, tiles_per_row, width, taps, h_stride, mode)
   const int key = (in_dtype == PYLON_F32 ? 4 : 0) | (w_dtype == PYLON_F32 ? 2 : 0) | (out_dtype == PYLON_F32 ? 1 : 0);
   switch (key) {
     case 0: GO(bf16_t, bf16_t, bf16_t); break;

@@ -213,7 +213,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     out: Optional[torch.Tensor] = None, rel: Optional[torch.Tensor] = None,
                     bucket: Optional[torch.Tensor] = None, sink: bool = False,
                     v_transposed: bool = False, chunk: Optional[int] = None,
-                    log_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    log_bias: Optional[torch.Tensor] = None, softcap: Optional[float] = None,
+                    sink_logit: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention of each token over its request's cached keys ``<=`` its position (with
     ``window`` the last so many, with ``chunk`` those of its own chunk: :func:`mask_code`).
     ``q`` is ``[tokens, heads, head_dim]`` and may be a slice of wider rows (a fused
@@ -221,9 +222,15 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     with ``bucket`` (int32 ``[n]``) adds ``rel[bucket[min(i - j, n - 1)], head]`` to the scaled
     score of query ``i`` and key ``j``; ``log_bias`` (float32 ``[2, heads]``: ``a`` then ``b``) takes
     ``a[head] * log(1 + b[head] * (i - j))`` off it instead; ``sink`` adds one to the softmax's
-    denominator.  With ``v_transposed`` the values lie as ``[pages, kv_heads, v_dim, page_size]``."""
+    denominator.  With ``v_transposed`` the values lie as ``[pages, kv_heads, v_dim, page_size]``.
+    ``softcap``: the scaled score ``s`` becomes ``softcap * tanh(s / softcap)``.  ``sink_logit``
+    (float32 ``[heads]``): ``exp(sink_logit[head])`` joins the denominator, unscaled and uncapped."""
     if q.dim() != 3:
         raise KernelError("paged_attention takes q as [tokens, heads, head_dim]")
+    if sink_logit is not None and (sink or sink_logit.shape != (q.shape[1],)):
+        raise KernelError("paged_attention: sink_logit is float32 [heads], and not together with the fixed sink")
+    if softcap is not None and not softcap > 0:
+        raise KernelError("paged_attention: a soft cap is positive")
     tokens, n_heads, head_dim = q.shape
     if v_transposed and v_cache.dim() == 4:
         v_shape = (v_cache.shape[0], v_cache.shape[3], v_cache.shape[1], v_cache.shape[2])
@@ -265,7 +272,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
               _dev(positions, "positions", torch.int32), tokens, n_heads, n_kv_heads, head_dim,
               page_size, mask_code(window, chunk), float(scale), v_dim, q.stride(0) if tokens > 1 else n_heads * head_dim,
               _dev(rel, "rel", torch.float32), _dev(bucket, "bucket", torch.int32),
-              0 if bucket is None else bucket.numel(), 1 if sink else 0, 1 if v_transposed else 0, _stream())
+              0 if bucket is None else bucket.numel(), 1 if sink else 0, 1 if v_transposed else 0,
+              float(softcap or 0.0), _dev(sink_logit, "sink_logit", torch.float32), _stream())
     return out
 
 
@@ -477,12 +485,18 @@ def add_bias_(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
     return x
 
 
+CONV_MODES = {"residual": 0, "silu": 1}
+
+
 def short_conv(h: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tensor], row_start: torch.Tensor,
-               row_slots: torch.Tensor, *, rows: int, max_count: int, out_dtype: torch.dtype) -> torch.Tensor:
+               row_slots: torch.Tensor, *, rows: int, max_count: int, out_dtype: torch.dtype,
+               mode: str = "residual") -> torch.Tensor:
     """``h[t] + sum_j weight[:, j] * h[t - taps + 1 + j]`` per channel and request, zeros before a
     request's start.  ``state`` (float32 ``[slots, taps - 1, width]``) holds every request's last
-    ``taps - 1`` inputs and is brought up to date; ``max_count`` bounds the tokens of a row."""
-    if h.dim() != 2 or weight.dim() != 2 or weight.shape[0] != h.shape[1]:
+    ``taps - 1`` inputs and is brought up to date; ``max_count`` bounds the tokens of a row.
+    ``mode="silu"``: ``silu`` of the convolution alone, without the input added.  ``h`` may be
+    the first columns of wider rows."""
+    if h.dim() != 2 or weight.dim() != 2 or weight.shape[0] != h.shape[1] or h.stride(1) != 1:
         raise KernelError("short_conv takes h [tokens, width] and weight [width, taps]")
     tokens, width = h.shape
     taps = weight.shape[1]
@@ -491,10 +505,10 @@ def short_conv(h: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tens
     if row_start.numel() != rows + 1 or row_slots.numel() != rows:
         raise KernelError("short_conv: one start per row and one more, and one slot per row")
     out = torch.empty((tokens, width), dtype=out_dtype, device=h.device)
-    _lib.call("pylon_short_conv", _dev(out, "out"), dtype_code(out_dtype), _dev(h, "h"), dtype_code(h.dtype),
+    _lib.call("pylon_short_conv", _dev(out, "out"), dtype_code(out_dtype), h.data_ptr(), dtype_code(h.dtype),
               _dev(weight, "weight"), dtype_code(weight.dtype), _dev(state, "state", torch.float32),
               _dev(row_start, "row_start", torch.int32), _dev(row_slots, "row_slots", torch.int32), rows,
-              int(max_count), width, taps, _stream())
+              int(max_count), width, taps, h.stride(0) if tokens > 1 else width, CONV_MODES[mode], _stream())
     return out
 
 
@@ -624,6 +638,91 @@ def qkv_bias_store(proj: torch.Tensor, bias: Optional[torch.Tensor], k_cache: Op
               _dev(slot_map if store else None, "slot_map", torch.int32), tokens, q_size, k_size, v_size,
               page_size, 1 if store else 0, _stream())
     return q
+
+
+def sigmoid_gate_(x: torch.Tensor, gate: torch.Tensor, *, per: int) -> torch.Tensor:
+    """``x[t, i] *= sigmoid(gate[t, i // per])`` in place: ``x`` contiguous ``[tokens, n]``, ``gate``
+    ``[tokens, n // per]`` of the same type (maybe columns of wider rows); ``per`` is a head's size
+    for one gate per head, 1 for one per element."""
+    if x.dim() != 2 or not x.is_contiguous() or gate.dim() != 2 or gate.stride(1) != 1 or gate.dtype != x.dtype:
+        raise KernelError("sigmoid_gate_ takes a contiguous [tokens, n] and gates of its type")
+    tokens, n = x.shape
+    if per < 1 or n % per or gate.shape != (tokens, n // per):
+        raise KernelError(f"sigmoid_gate_: {n} elements in groups of {per} need gates [tokens, {n // max(per, 1)}]")
+    _lib.call("pylon_sigmoid_gate", _dev(x, "x"), dtype_code(x.dtype), gate.data_ptr(),
+              gate.stride(0) if tokens > 1 else n // per, tokens, n, int(per), _stream())
+    return x
+
+
+def scaled_sum(a: torch.Tensor, a_scale: float, b: torch.Tensor, b_scale: float) -> torch.Tensor:
+    """``a_scale * a + b_scale * b`` as float32 ``[tokens, dim]``; ``a`` and ``b`` are each
+    ``[tokens, dim]`` or a stack ``[parts, tokens, dim]`` of float32 partial sums still to be added up."""
+    shape = tuple(a.shape[-2:])
+    for t in (a, b):
+        if t.dim() not in (2, 3) or tuple(t.shape[-2:]) != shape or not t.is_contiguous():
+            raise KernelError("scaled_sum takes two contiguous [tokens, dim] tensors or stacks of such")
+        if t.dim() == 3 and t.dtype != torch.float32:
+            raise KernelError("scaled_sum: a stack of partial sums is float32")
+    out = torch.empty(shape, dtype=torch.float32, device=a.device)
+    _lib.call("pylon_scaled_sum", _dev(out, "out"), _dev(a, "a"), dtype_code(a.dtype), a.shape[0] if a.dim() == 3 else 1,
+              float(a_scale), _dev(b, "b"), dtype_code(b.dtype), b.shape[0] if b.dim() == 3 else 1, float(b_scale),
+              out.numel(), _stream())
+    return out
+
+
+def delta_rule_ok(dim: int, vdim: int) -> bool:
+    """Whether :func:`delta_rule` has a layout for heads of ``dim x vdim`` (the kernel's own rule)."""
+    p = 1
+    while p * 2 <= 64 and p * 2 <= dim and vdim * p * 2 <= 256:
+        p *= 2
+    r = -(-dim // p)
+    while r > 64 and p * 2 <= 64 and vdim * p * 2 <= 1024:
+        p *= 2
+        r = -(-dim // p)
+    return dim >= 1 and vdim >= 1 and r <= 128 and vdim * p <= 1024 and (r <= 64 or vdim * p <= 256)
+
+
+def delta_rule(qkv: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, a_log: torch.Tensor,
+               dt_bias: torch.Tensor, norm_weight: torch.Tensor, row_start: torch.Tensor, row_slots: torch.Tensor, *,
+               rows: int, heads: int, kv_heads: int, dim: int, vdim: int, gate_off: int, beta_off: int,
+               decay_off: int, eps: float, unit_eps: float, q_scale: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """The gated delta rule over the rows of a step: per request and head ``S <- g S; u = beta (v -
+    S^T k); S <- S + k u^T; o = S^T q``.  ``qkv`` float32 ``[tokens, 2 kv_heads dim + heads vdim]``
+    holds q, k and v (after their convolution and activation); q and k become unit vectors per head
+    (``unit_eps`` inside the root; q also times ``q_scale``).  ``proj`` float32 rows hold, from
+    ``gate_off``, the output gate ``[heads, vdim]``, and per head the logits of ``beta`` (from
+    ``beta_off``) and of the decay (from ``decay_off``): ``beta = sigmoid(b)``, ``g = exp(-exp(a_log) *
+    softplus(a + dt_bias))``.  ``state`` float32 ``[slots, heads, vdim, dim]`` (the state transposed)
+    is read and left up to date.  Returns ``o / rms(o) * norm_weight * silu(gate)`` as ``[tokens,
+    heads * vdim]``."""
+    if qkv.dim() != 2 or proj.dim() != 2 or qkv.dtype != torch.float32 or proj.dtype != torch.float32 \
+            or qkv.stride(1) != 1 or proj.stride(1) != 1 or qkv.shape[0] != proj.shape[0]:
+        raise KernelError("delta_rule takes float32 rows of q, k, v and of the projection, one per token")
+    tokens = qkv.shape[0]
+    qk = kv_heads * dim
+    if qkv.shape[1] < 2 * qk + heads * vdim:
+        raise KernelError("delta_rule: the rows of q, k and v are too short")
+    if max(gate_off + heads * vdim, beta_off + heads, decay_off + heads) > proj.shape[1] or min(gate_off, beta_off, decay_off) < 0:
+        raise KernelError("delta_rule: the gate, beta or the decay lie outside the projection's rows")
+    if state.dim() != 4 or state.shape[1:] != (heads, vdim, dim) or state.dtype != torch.float32 or not state.is_contiguous():
+        raise KernelError(f"delta_rule: state must be float32 [slots, {heads}, {vdim}, {dim}]")
+    if a_log.shape != (heads,) or dt_bias.shape != (heads,) or norm_weight.shape != (vdim,):
+        raise KernelError("delta_rule: one rate and one bias per head, one norm weight per value element")
+    if row_start.numel() != rows + 1 or row_slots.numel() != rows:
+        raise KernelError("delta_rule: one start per row and one more, and one slot per row")
+    if not delta_rule_ok(dim, vdim) or heads % kv_heads:
+        raise KernelError(f"delta_rule does not take {heads} heads over {kv_heads} of {dim} x {vdim}")
+    if not qkv.is_cuda:
+        raise KernelError("qkv must live on the GPU; there is no CPU path")
+    out = torch.empty((tokens, heads * vdim), dtype=out_dtype, device=qkv.device)
+    _lib.call("pylon_delta_rule", _dev(out, "out"), dtype_code(out_dtype), heads * vdim, qkv.data_ptr(),
+              qkv.stride(0) if tokens > 1 else qkv.shape[1], 0, qk, 2 * qk, proj.data_ptr(),
+              proj.stride(0) if tokens > 1 else proj.shape[1], int(gate_off), int(beta_off), int(decay_off),
+              _dev(a_log, "a_log", torch.float32), _dev(dt_bias, "dt_bias", torch.float32),
+              _dev(norm_weight, "norm_weight", torch.float32), _dev(state, "state", torch.float32),
+              _dev(row_start, "row_start", torch.int32), _dev(row_slots, "row_slots", torch.int32), rows, heads,
+              kv_heads, dim, vdim, float(eps), float(unit_eps), float(q_scale), _stream())
+    return out
 
 
 def gated_act(gate_up: torch.Tensor, *, alpha: float, offset: float, limit: float,
@@ -1152,24 +1251,32 @@ def qkv_prepare_wide(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: Optional[t
                      v_cache: Optional[torch.Tensor], *, n_heads: int, n_kv_heads: int, head_dim: int, v_dim: int,
                      q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
                      inv_freq: Optional[torch.Tensor], rot_dim: int, interleaved: bool,
-                     positions: Optional[torch.Tensor], slot_map: Optional[torch.Tensor], store_kv: bool) -> None:
+                     positions: Optional[torch.Tensor], slot_map: Optional[torch.Tensor], store_kv: bool,
+                     per_head: bool = False, rot_scale: float = 1.0, values_from_keys: bool = False) -> None:
     """q/k/v preparation with norms over whole projections: ``q_weight`` (float32, all heads of q
     side by side) and ``k_weight`` norm the whole q row and the whole k row of a token (None: no
     norm); the first ``rot_dim`` elements of every head of q and k are rotated by ``position *
     inv_freq[i]``, pairing neighbours (``interleaved``) or halves; q goes to ``q_out``, k and v
-    (heads of ``v_dim`` elements) into the tokens' cache slots."""
+    (heads of ``v_dim`` elements) into the tokens' cache slots.  ``per_head``: the norms run head
+    by head with weights of ``head_dim`` elements.  ``rot_scale`` multiplies every cosine and
+    sine.  ``values_from_keys``: there are no value columns; the values are the keys as projected,
+    before norm and rotation (``v_dim`` is then ``head_dim``).  The rows of ``qkv`` may be wider
+    than q, k and v together (further columns of a fused projection are left alone)."""
     if qkv.dim() != 2 or qkv.stride(1) != 1:
         raise KernelError("qkv_prepare_wide takes a 2-D projection output with contiguous rows")
     tokens, width = qkv.shape
     q_size, k_size, v_size = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * v_dim
-    if width != q_size + (k_size + v_size if store_kv else 0):
+    if values_from_keys and v_dim != head_dim:
+        raise KernelError("qkv_prepare_wide: values that are the keys have the keys' size")
+    v_offset = q_size if values_from_keys else q_size + k_size
+    if width < q_size + (max(k_size, v_offset - q_size + v_size) if store_kv else 0):
         raise KernelError(f"qkv_prepare_wide: projection width {width} does not match the heads")
     if q_out.shape != (tokens, n_heads, head_dim) or q_out.dtype != qkv.dtype:
         raise KernelError("qkv_prepare_wide: q_out has the wrong shape or dtype")
-    if q_weight is not None and q_weight.shape != (q_size,):
-        raise KernelError(f"qkv_prepare_wide: q_weight must have shape ({q_size},)")
-    if k_weight is not None and k_weight.shape != (k_size,):
-        raise KernelError(f"qkv_prepare_wide: k_weight must have shape ({k_size},)")
+    if q_weight is not None and q_weight.shape != ((head_dim,) if per_head else (q_size,)):
+        raise KernelError(f"qkv_prepare_wide: q_weight must have shape ({head_dim if per_head else q_size},)")
+    if k_weight is not None and k_weight.shape != ((head_dim,) if per_head else (k_size,)):
+        raise KernelError(f"qkv_prepare_wide: k_weight must have shape ({head_dim if per_head else k_size},)")
     if rot_dim and (inv_freq is None or inv_freq.numel() != rot_dim // 2 or positions is None
                     or positions.numel() != tokens):
         raise KernelError("qkv_prepare_wide: a rotation needs rot_dim/2 frequencies and one position per token")
@@ -1187,7 +1294,8 @@ def qkv_prepare_wide(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: Optional[t
               _dev(q_weight, "q_weight", torch.float32), _dev(k_weight, "k_weight", torch.float32), float(eps),
               _dev(inv_freq, "inv_freq", torch.float32), int(rot_dim), 1 if interleaved else 0,
               _dev(positions, "positions", torch.int32), _dev(slot_map if store_kv else None, "slot_map", torch.int32),
-              tokens, n_heads, n_kv_heads, head_dim, v_dim, 1 if store_kv else 0, _stream())
+              tokens, n_heads, n_kv_heads, head_dim, v_dim, 1 if store_kv else 0, 1 if per_head else 0,
+              float(rot_scale), int(v_offset), _stream())
 
 
 def latent_prepare(down: torch.Tensor, cache: Optional[torch.Tensor], slot_map: Optional[torch.Tensor], *,
@@ -1250,12 +1358,16 @@ def head_project(x: torch.Tensor, m: torch.Tensor, *, gate: Optional[torch.Tenso
     return out
 
 
+ROUTE_SCORINGS = {"top_softmax": 0, "sigmoid": 1}
+
+
 def route_top(logits: torch.Tensor, bias: Optional[torch.Tensor], *, n_experts: int, top: int,
-              shared_gate: bool):
+              shared_gate: bool, scoring: str = "top_softmax"):
     """From float32 router logits ``[tokens, n_experts (+ 1 with shared_gate)]``: the ``top``
     experts with the largest ``logit + bias`` per token (int32 ``[tokens, top]``, the lower index
     among equals), the softmax over those alone (float32 ``[tokens, top]``), and ``sigmoid`` of the
-    last column (float32 ``[tokens]``, or None)."""
+    last column (float32 ``[tokens]``, or None).  ``scoring="sigmoid"``: the weights are the chosen
+    experts' own ``sigmoid(logit + bias)``, as they are."""
     if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1:
         raise KernelError("route_top takes float32 logits [tokens, experts]")
     tokens = logits.shape[0]
@@ -1268,7 +1380,7 @@ def route_top(logits: torch.Tensor, bias: Optional[torch.Tensor], *, n_experts: 
     gate = torch.empty((tokens,), dtype=torch.float32, device=logits.device) if shared_gate else None
     _lib.call("pylon_route_top", _dev(experts, "experts"), _dev(weights, "weights"), _dev(gate, "gate"),
               logits.data_ptr(), logits.stride(0), _dev(bias, "bias", torch.float32), tokens, n_experts, top,
-              _stream())
+              ROUTE_SCORINGS[scoring], _stream())
     return experts, weights, gate
 
 
@@ -1300,14 +1412,19 @@ EXPERT_ACTS = {"silu_gated": 0, "relu2": 1}  # silu(W_gate x) * (W_up x); relu(W
 
 
 def expert_gate_up(x: torch.Tensor, gate_up: torch.Tensor, experts: torch.Tensor, *, n_experts: int,
-                   ff: int, act: str = "silu_gated") -> torch.Tensor:
+                   ff: int, act: str = "silu_gated", input_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``silu(W_gate[e] x_t) * (W_up[e] x_t)`` for every token and each of its chosen experts:
     ``gate_up`` is ``[n_experts * 2 ff, width]`` (an expert's gate rows, then its up rows);
     returns ``[tokens * top, ff]`` of ``x``'s type, float sums rounded once.  ``act="relu2"``: plain
     experts, ``relu(W_up[e] x_t)^2`` with the matrix ``[n_experts * ff, width]``.  A choice of
-    ``n_experts`` or more (an identity) is passed over: its rows of the result are not written."""
+    ``n_experts`` or more (an identity) is passed over: its rows of the result are not written.
+    ``input_weights`` (float32 ``[tokens, top]``): a choice's expert works on ``x_t`` times the
+    choice's weight (formed in float32)."""
     tokens, width = x.shape
     top = experts.shape[1]
+    if input_weights is not None and (input_weights.shape != (tokens, top) or input_weights.dtype != torch.float32
+                                      or not input_weights.is_contiguous()):
+        raise KernelError("expert_gate_up: input_weights must be float32 [tokens, top]")
     per_expert = 2 * ff if act == "silu_gated" else ff
     if gate_up.shape != (n_experts * per_expert, width) or gate_up.stride(1) != 1 or x.stride(1) != 1:
         raise KernelError(f"expert_gate_up: the experts' matrix must be [experts * {per_expert}, width]")
@@ -1316,7 +1433,7 @@ def expert_gate_up(x: torch.Tensor, gate_up: torch.Tensor, experts: torch.Tensor
     hidden = torch.empty((tokens * top, ff), dtype=x.dtype, device=x.device)
     _lib.call("pylon_expert_gate_up", _dev(hidden, "hidden"), x.data_ptr(), dtype_code(x.dtype), x.stride(0),
               gate_up.data_ptr(), dtype_code(gate_up.dtype), gate_up.stride(0), _dev(experts, "experts"), tokens, top,
-              ff, width, EXPERT_ACTS[act], n_experts, _stream())
+              ff, width, EXPERT_ACTS[act], n_experts, _dev(input_weights, "input_weights", torch.float32), _stream())
     return hidden
 
 
@@ -1371,14 +1488,17 @@ def experts_grouped_ok(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tenso
 def experts_grouped(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, experts: torch.Tensor,
                     weights: torch.Tensor, *, n_experts: int, ff: int, shared: Optional[torch.Tensor] = None,
                     shared_gate: Optional[torch.Tensor] = None, act: str = "silu_gated",
-                    identity_weight: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    identity_weight: Optional[torch.Tensor] = None, weight_on_input: bool = False) -> torch.Tensor:
     """What :func:`expert_gate_up` and :func:`expert_down` compute, for many bfloat16 tokens: the
     (token, choice) pairs are sorted by expert on the device (nothing is read back), every expert's
     pairs go through its gate/up and its down matrix as tiles of 64 rows on the matrix cores, and
     the results return to their tokens weighted, in the order of the token's choices.  float32
     ``[tokens, width]``.  ``act`` as for :func:`expert_gate_up`.  Choices of ``n_experts`` or more
     (identity experts) sort behind every expert's pairs and run through no matrix; with
-    ``identity_weight`` (float32 ``[tokens]``) ``identity_weight[t] * x[t]`` is added for them."""
+    ``identity_weight`` (float32 ``[tokens]``) ``identity_weight[t] * x[t]`` is added for them.
+    ``weight_on_input``: a choice's weight multiplies its expert's input instead of its output
+    (gated experts: the gate's and the up's float32 sums are scaled before the activation, which
+    is the product of the scaled input because the two products are linear)."""
     tokens, width = x.shape
     top = experts.shape[1]
     pairs = tokens * top
@@ -1394,9 +1514,15 @@ def experts_grouped(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, 
     rows = (order // top).to(torch.int32)  # sorted place -> token
     place = torch.empty_like(order).scatter_(0, order, torch.arange(pairs, device=x.device)).to(torch.int32)
     hidden = torch.empty((pairs, ff), dtype=torch.bfloat16, device=x.device)
+    row_scale = None
+    if weight_on_input:
+        if act != "silu_gated":
+            raise KernelError("experts_grouped: weights on the input go with gated experts")
+        row_scale = weights.reshape(-1)[order].contiguous()  # sorted place -> the pair's weight
+        weights = torch.ones_like(weights)
     _lib.call("pylon_grouped_gate_up", _dev(hidden, "hidden"), x.data_ptr(), x.stride(0), _dev(rows, "rows"),
               gate_up.data_ptr(), gate_up.stride(0), _dev(offsets, "offsets"), pairs, n_experts, ff, width, tokens,
-              EXPERT_ACTS[act], _stream())
+              EXPERT_ACTS[act], _dev(row_scale, "row_scale", torch.float32), _stream())
     y = torch.empty((pairs, width), dtype=torch.float32, device=x.device)
     _lib.call("pylon_grouped_down", _dev(y, "y"), _dev(hidden, "hidden"), ff, down.data_ptr(), down.stride(0),
               _dev(offsets, "offsets"), pairs, n_experts, ff, width, _stream())

@@ -1,2 +1,2 @@
 """Built-in model families; importing this package registers them."""
-from . import gimudra, qwen3, pavitar, vupuzen  # noqa: F401
+from . import gimudra, qwen3, pavitar, tukarax, vupuzen  # noqa: F401

@@ -12,6 +12,13 @@ projection (``qk_norm_over="projection"``), for a rotation that pairs neighbouri
 position part's ``interleaved``) over a part of the head, for values of another size than keys,
 and for keys visible inside the query's chunk of positions only (``chunk``); these go through
 :func:`ops.qkv_prepare_wide` and the same attention kernels, which take the mask as one integer.
+
+Further options of the spec: a rotation whose frequencies are stretched for long contexts and
+whose cosines and sines carry a factor (the position part's ``rot_scale``); scores capped by
+``softcap * tanh(s / softcap)``; a learned sink per head in the softmax's denominator; values that
+are the keys as projected (``values_from_keys``: no value projection); and an output gate
+``sigmoid(W_g h)`` per head or per element on the heads' outputs, whose rows are the last of the
+fused projection ``[q; k; v; g]``.  Capped scores and the learned sink run on the general kernel.
 """
 from __future__ import annotations
 
@@ -31,7 +38,8 @@ class Attention(Part):
         if spec.n_heads % spec.n_kv_heads:
             raise ValueError("The number of Q heads must be divisible by the number of KV heads.")
         per_head = (not spec.qk_norm or spec.qk_norm_over == "head") and not getattr(spec.position, "interleaved", False) \
-            and spec.value_dim == spec.head_dim
+            and spec.value_dim == spec.head_dim and not spec.values_from_keys and spec.output_gate is None \
+            and getattr(spec.position, "scaling", None) is None
         if per_head and (spec.head_dim % 16 or not 16 <= spec.head_dim <= 512):
             raise ValueError(
                 f"head_dim {spec.head_dim} is not supported: the attention kernels take "
@@ -47,10 +55,21 @@ class Attention(Part):
             raise ValueError(f"qk_norm_over must be 'head' or 'projection', got {spec.qk_norm_over!r}")
         if spec.value_dim < 1 or spec.value_dim > 512:
             raise ValueError(f"value heads of {spec.value_dim} elements are not supported: 1 to 512")
+        if spec.output_gate not in (None, "head", "element"):
+            raise ValueError(f"output_gate must be None, 'head' or 'element', got {spec.output_gate!r}")
+        if spec.values_from_keys and spec.value_dim != spec.head_dim:
+            raise ValueError("values that are the keys have the keys' size")
+        if spec.softcap is not None and not spec.softcap > 0:
+            raise ValueError("a soft cap of the scores is positive")
         self.spec = spec
         self.dtype = dtype
         q, kv = spec.q_size, spec.kv_size
-        self.add_param("qkv", (q + kv + spec.v_size, spec.hidden_size), dtype, device)
+        # rows of the fused projection: q, k, v (none when the values are the keys), the gate
+        self.v_rows = 0 if spec.values_from_keys else spec.v_size
+        self.gate_off = q + kv + self.v_rows
+        self.add_param("qkv", (self.gate_off + spec.gate_size, spec.hidden_size), dtype, device)
+        if spec.sink:
+            self.add_param("sink", (spec.n_heads,), torch.float32, device, role="vector")
         self.add_param("out", (spec.hidden_size, spec.n_heads * spec.value_dim), dtype, device)
         if spec.qk_norm:
             over_heads = spec.qk_norm_over == "head"
@@ -60,7 +79,10 @@ class Attention(Part):
         # what the per-head preparation kernels (and the decode kernel that prepares its own
         # operands) cover: norms head by head, halves rotated together, values as large as keys
         self.plain = ((not spec.qk_norm or spec.qk_norm_over == "head") and spec.value_dim == spec.head_dim
-                      and not getattr(self.position, "interleaved", False))
+                      and not getattr(self.position, "interleaved", False) and not spec.values_from_keys
+                      and spec.output_gate is None and getattr(self.position, "rot_scale", 1.0) == 1.0)
+        # capped scores and a learned sink: the general attention kernel
+        self.special = spec.softcap is not None or spec.sink
 
     def cache_requirement(self) -> KVRequirement:
         spec = self.spec
@@ -83,11 +105,11 @@ class Attention(Part):
         spec = self.spec
         tokens = h.shape[0]
         weight = self.params["qkv"]
-        if not stores:
+        if not stores and spec.output_gate is None:
             weight = weight[: spec.q_size]
         rotary = self.position.rotary()
         mask = dict(window=spec.window, chunk=spec.chunk)
-        if self.plain and spec.chunk is None and ctx.decode_only and cache.k is not None and ops.decode_fused_ok(
+        if self.plain and not self.special and spec.chunk is None and ctx.decode_only and cache.k is not None and ops.decode_fused_ok(
                 self.dtype, cache.k, tokens=tokens, n_heads=spec.n_heads, head_dim=spec.head_dim,
                 rot_dim=rotary[1] if rotary else 0):
             # one launch adds the projection's partial sums if it comes as such, norms and
@@ -123,8 +145,11 @@ class Attention(Part):
                 inv_freq=rotary[0] if rotary else None, rot_dim=rotary[1] if rotary else 0,
                 interleaved=getattr(self.position, "interleaved", False),
                 positions=ctx.positions, slot_map=cache.slot_map, store_kv=stores,
+                per_head=spec.qk_norm and spec.qk_norm_over == "head",
+                rot_scale=getattr(self.position, "rot_scale", 1.0), values_from_keys=spec.values_from_keys,
             )
-        same_size = spec.value_dim == spec.head_dim  # the matrix-core kernels take values as large as keys
+        # the matrix-core kernels take values as large as keys, plain scores and no sink
+        same_size = spec.value_dim == spec.head_dim and not self.special
         if same_size and ctx.decode_only and ops.decode_attention_ok(q, cache.k):
             cuts, splits = ops.decode_launch(tokens, spec.n_kv_heads, self._span(ctx))
             # in a decode-only step token t is row t
@@ -160,10 +185,14 @@ class Attention(Part):
         else:
             context = ops.paged_attention(
                 q, cache.k, cache.v, cache.block_table, ctx.tok_row, ctx.positions,
-                page_size=cache.page_size, scale=spec.scale, **mask,
+                page_size=cache.page_size, scale=spec.scale, softcap=spec.softcap,
+                sink_logit=self.params.get("sink"), **mask,
             )
-        return ops.linear_for_residual(context.view(tokens, spec.n_heads * spec.value_dim), self.params["out"],
-                                       out_dtype=self.dtype)
+        context = context.view(tokens, spec.n_heads * spec.value_dim)
+        if spec.output_gate is not None:
+            ops.sigmoid_gate_(context, qkv[:, self.gate_off: self.gate_off + spec.gate_size],
+                              per=spec.value_dim if spec.output_gate == "head" else 1)
+        return ops.linear_for_residual(context, self.params["out"], out_dtype=self.dtype)
 
 
 def distance_buckets(rows: int, far: float) -> list:

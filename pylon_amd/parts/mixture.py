@@ -19,6 +19,12 @@ matrix ``up`` in place of ``gate_up``), and for the other way of routing (``scor
 only, a choice limited to the best groups of neighbouring outputs, weights that are the scores times a
 constant, and identity experts (router outputs without matrices, whose output is the input itself:
 the expert kernels pass over them and add the input times the sum of their weights).
+
+``scoring="sigmoid"``: the chosen experts' weights are the sigmoids of their own router outputs, not
+renormalised.  ``weight_on_input``: a chosen expert runs on the token's input times its weight,
+``sum_e expert_e(w_e h)``; the token-by-token kernel scales the input in float32 as it stages it, the
+sorted path scales the gate's and the up's float32 sums before the activation (the same number,
+because the two products are linear).
 """
 from __future__ import annotations
 
@@ -42,10 +48,12 @@ class MixtureFeedForward(Part):
             raise ValueError("a gate of the shared expert needs a shared expert")
         if spec.expert_act not in ops.EXPERT_ACTS:
             raise ValueError(f"unknown activation of the experts {spec.expert_act!r} (known: {', '.join(ops.EXPERT_ACTS)})")
-        if spec.scoring not in ("top_softmax", "softmax_all"):
-            raise ValueError(f"unknown scoring {spec.scoring!r} (known: top_softmax, softmax_all)")
+        if spec.scoring not in ("top_softmax", "softmax_all", "sigmoid"):
+            raise ValueError(f"unknown scoring {spec.scoring!r} (known: top_softmax, softmax_all, sigmoid)")
+        if spec.weight_on_input and (spec.expert_act != "silu_gated" or spec.n_identity):
+            raise ValueError("weights on the experts' inputs go with gated experts and without identity experts")
         outputs = spec.n_experts + spec.n_identity
-        if spec.scoring == "top_softmax":
+        if spec.scoring in ("top_softmax", "sigmoid"):
             if spec.n_identity or spec.groups != 1 or spec.route_scale != 1.0:
                 raise ValueError("identity experts, groups and a scale of the weights belong to the scoring softmax_all")
         else:
@@ -91,7 +99,7 @@ class MixtureFeedForward(Part):
         else:
             experts, weights, shared_gate = ops.route_top(
                 logits, self.params.get("router_bias"), n_experts=spec.n_experts, top=spec.top,
-                shared_gate=spec.shared_gate)
+                shared_gate=spec.shared_gate, scoring=spec.scoring)
         first = self.params["gate_up"] if self.gated else self.params["up"]
         shared = None
         if spec.shared_size is not None:
@@ -101,9 +109,12 @@ class MixtureFeedForward(Part):
             # many tokens: sorted by expert, every expert's tokens as tiles on the matrix cores
             return ops.experts_grouped(h, first, self.params["down"], experts, weights,
                                        n_experts=spec.n_experts, ff=spec.expert_size, shared=shared,
-                                       shared_gate=shared_gate, act=spec.expert_act, identity_weight=identity)
+                                       shared_gate=shared_gate, act=spec.expert_act, identity_weight=identity,
+                                       weight_on_input=spec.weight_on_input)
         hidden = ops.expert_gate_up(h, first, experts, n_experts=spec.n_experts, ff=spec.expert_size,
-                                    act=spec.expert_act)
+                                    act=spec.expert_act, input_weights=weights if spec.weight_on_input else None)
+        if spec.weight_on_input:
+            weights = torch.ones_like(weights)  # the weights went in with the inputs
         return ops.expert_down(hidden, self.params["down"], experts, weights, n_experts=spec.n_experts,
                                width=spec.hidden_size, shared=shared, shared_gate=shared_gate,
                                identity_x=h if identity is not None else None, identity_weight=identity)

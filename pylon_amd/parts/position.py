@@ -27,7 +27,10 @@ class RotaryPosition(Part):
             raise ValueError("rotary_dim must be even and at least 2")
         self.spec = spec
         self.interleaved = spec.interleaved
-        if spec.interleaved:
+        self.rot_scale = 1.0  # what every cosine and sine is multiplied by
+        if spec.scaling is not None:
+            inv_freq, self.rot_scale = scaled_frequencies(spec)
+        elif spec.interleaved:
             # neighbours (2i, 2i + 1) turn together; frequencies theta ** (-2i/d) formed in double
             # precision and rounded to float32 once
             exponents = torch.arange(0, spec.rotary_dim, 2, dtype=torch.float64) / spec.rotary_dim
@@ -41,11 +44,34 @@ class RotaryPosition(Part):
         return self.inv_freq, self.spec.rotary_dim
 
 
+def scaled_frequencies(spec: PositionSpec):
+    """``(float32 frequencies of the rotary_dim / 2 pairs, the factor on cosine and sine)`` of a
+    rotation whose slow pairs are stretched by ``spec.scaling`` (:class:`RotaryScalingSpec`);
+    formed in double precision and rounded once."""
+    import math
+
+    sc, dims = spec.scaling, spec.rotary_dim
+    if not (sc.factor >= 1.0 and sc.original > 0 and sc.fast > 0 and sc.slow > 0 and spec.theta > 1.0):
+        raise ValueError("a scaled rotation needs factor >= 1 and positive original, fast and slow")
+
+    def where(turns: float) -> float:
+        return dims * math.log(sc.original / (2.0 * math.pi * turns)) / (2.0 * math.log(spec.theta))
+
+    lo = max(math.floor(where(sc.fast)), 0)
+    hi = min(math.ceil(where(sc.slow)), dims - 1)
+    index = torch.arange(dims // 2, dtype=torch.float64)
+    plain = torch.tensor(spec.theta, dtype=torch.float64) ** (-2.0 * index / dims)
+    ramp = ((index - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    freq = plain / sc.factor * ramp + plain * (1.0 - ramp)
+    return freq.to(torch.float32), 0.1 * math.log(sc.factor) + 1.0
+
+
 class NoPosition(Part):
     def __init__(self, spec: PositionSpec, *, dtype: torch.dtype, device) -> None:
         super().__init__()
         self.spec = spec
         self.interleaved = False
+        self.rot_scale = 1.0
 
     def rotary(self):
         return None
