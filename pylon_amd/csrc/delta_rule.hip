@@ -20,8 +20,8 @@
 
 #define DR_PAD 4  // floats between two slices of q or k in LDS (keeps the slices' reads off one bank)
 
-template <int RT, typename TO>
-__global__ void __launch_bounds__(RT > 64 ? 256 : 1024)
+template <int RT, int MAXT, typename TO>
+__global__ void __launch_bounds__(MAXT)
 delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __restrict__ qkv, long long qkv_stride,
                   int q_off, int k_off, int v_off, const float* __restrict__ proj, long long proj_stride, int g_off,
                   int b_off, int a_off, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
@@ -87,26 +87,26 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
       for (int i = 0; i < n; ++i) {
         const float4* k4 = reinterpret_cast<const float4*>(ks + i * KS + p * (RT + DR_PAD));
         const float4* q4 = reinterpret_cast<const float4*>(qs + i * KS + p * (RT + DR_PAD));
-        float kk[RT];
+        float a = 0.f;
 #pragma unroll
         for (int r = 0; r < RT / 4; ++r) {
           const float4 v = k4[r];
-          kk[4 * r] = v.x, kk[4 * r + 1] = v.y, kk[4 * r + 2] = v.z, kk[4 * r + 3] = v.w;
+          a = fmaf(S[4 * r], v.x, a);
+          a = fmaf(S[4 * r + 1], v.y, a);
+          a = fmaf(S[4 * r + 2], v.z, a);
+          a = fmaf(S[4 * r + 3], v.w, a);
         }
-        float a = 0.f;
-#pragma unroll
-        for (int r = 0; r < RT; ++r) a = fmaf(S[r], kk[r], a);
         for (int off = P >> 1; off > 0; off >>= 1) a += __shfl_xor(a, off, PYLON_WAVE);
         const float g = decays[i];
         const float u = betas[i] * (vs[i * vdim + j] - g * a);
         float o = 0.f;
 #pragma unroll
         for (int r = 0; r < RT / 4; ++r) {
-          const float4 v = q4[r];
-          const float qq[4] = {v.x, v.y, v.z, v.w};
+          const float4 v = q4[r], w = k4[r];  // the keys once more from LDS: cheaper than holding them
+          const float qq[4] = {v.x, v.y, v.z, v.w}, kk[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
-            S[4 * r + c] = fmaf(kk[4 * r + c], u, g * S[4 * r + c]);
+            S[4 * r + c] = fmaf(kk[c], u, g * S[4 * r + c]);
             o = fmaf(S[4 * r + c], qq[c], o);
           }
         }
@@ -188,18 +188,23 @@ extern "C" int pylon_delta_rule(void* out, int out_dtype, long long out_stride, 
   const int threads = (vdim * P + PYLON_WAVE - 1) / PYLON_WAVE * PYLON_WAVE;
   PYLON_REQUIRE(static_cast<long long>(rows) * heads < (1ll << 31), "delta_rule: too many rows");
   dim3 grid(static_cast<unsigned>(rows * heads)), block(threads);
-#define GO(RTV, TO)                                                                                                \
-  hipLaunchKernelGGL((delta_rule_kernel<RTV, TO>), grid, block, lds, stream, (TO*)out, out_stride, qkv, qkv_stride, \
-                     q_off, k_off, v_off, proj, proj_stride, g_off, b_off, a_off, a_log, dt_bias, norm_w, state,    \
-                     row_start, row_slots, heads, kv_heads, dim, vdim, P, R, CT, eps, unit_eps, q_scale)
-#define PICK(TO)                    \
-  switch (RT) {                     \
-    case 4: GO(4, TO); break;       \
-    case 8: GO(8, TO); break;       \
-    case 16: GO(16, TO); break;     \
-    case 32: GO(32, TO); break;     \
-    case 64: GO(64, TO); break;     \
-    default: GO(128, TO); break;    \
+#define GO(RTV, MAXT, TO)                                                                                     \
+  hipLaunchKernelGGL((delta_rule_kernel<RTV, MAXT, TO>), grid, block, lds, stream, (TO*)out, out_stride, qkv,   \
+                     qkv_stride, q_off, k_off, v_off, proj, proj_stride, g_off, b_off, a_off, a_log, dt_bias,   \
+                     norm_w, state, row_start, row_slots, heads, kv_heads, dim, vdim, P, R, CT, eps, unit_eps,  \
+                     q_scale)
+  // up to 256 threads a workgroup may use all registers of a lane; more threads share them
+#define BOTH(RTV, TO)                     \
+  if (threads <= 256) GO(RTV, 256, TO);   \
+  else GO(RTV, 1024, TO)
+#define PICK(TO)                         \
+  switch (RT) {                          \
+    case 4: BOTH(4, TO); break;          \
+    case 8: BOTH(8, TO); break;          \
+    case 16: BOTH(16, TO); break;        \
+    case 32: BOTH(32, TO); break;        \
+    case 64: BOTH(64, TO); break;        \
+    default: GO(128, 256, TO); break;    \
   }
   if (out_dtype == PYLON_F32) {
     PICK(float);
@@ -207,6 +212,7 @@ extern "C" int pylon_delta_rule(void* out, int out_dtype, long long out_stride, 
     PICK(bf16_t);
   }
 #undef PICK
+#undef BOTH
 #undef GO
   PYLON_LAUNCHED("delta_rule");
 }

@@ -176,13 +176,18 @@ def parallel_mixer(h, m: dict, w: dict, pre: str, eps: float) -> np.ndarray:
 def route(h, router: np.ndarray, top: int):
     """``(chosen experts [n, top], their weights [n, top], margin [n])``: the scores are sigmoids of
     the router's outputs, the weights the chosen scores as they are; the margin is the distance
-    between the last score taken and the first left."""
-    s = sigmoid(h @ router.T)
+    between the last router output taken and the first left, as a share of the token's largest
+    output (outputs, not scores: where the sigmoid is flat, scores lie closer together than the
+    outputs that rounding moves; a share, because rounding moves an output by a share of its size)."""
+    z = h @ router.T
+    s = sigmoid(z)
     order = np.argsort(-s, axis=-1, kind="stable")
     chosen = order[:, :top]
     weights = np.take_along_axis(s, chosen, axis=-1)
     if s.shape[1] > top:
-        margin = weights[:, -1] - np.take_along_axis(s, order[:, top: top + 1], axis=-1)[:, 0]
+        margin = (np.take_along_axis(z, order[:, top - 1: top], axis=-1)
+                  - np.take_along_axis(z, order[:, top: top + 1], axis=-1))[:, 0]
+        margin = margin / np.maximum(np.abs(z).max(axis=-1), 1e-30)
     else:
         margin = np.full(h.shape[0], np.inf)
     return chosen, weights, margin
