@@ -2,7 +2,7 @@
 and uniform-random token ids, on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
-                    [--shape 4b|8b|32b] [--prompt-len N] [--design vupuzen|pavitar|gimudra [--beside qwen3|vupuzen|pavitar] [--design-shapes 8b,...]]
+                    [--shape 4b|8b|32b] [--prompt-len N] [--design vupuzen|pavitar|gimudra|tukarax [--beside qwen3|vupuzen|pavitar|gimudra] [--design-shapes 8b,...]]
 
 Everything goes the product's own way.  Start-up is ``Runner.from_random``: the fit check,
 the measured activation headroom, the page pool sized from the card's memory and the decode
@@ -355,6 +355,32 @@ def gimudra_json(shape: dict, layers: int) -> dict:
             "embedding": {"scale": 1.0}, "layers": out}
 
 
+def tukarax_json(shape: dict, layers: int) -> dict:
+    """A Tukarax configuration of the shape's layer sizes: parallel and attention layers in turns.
+    Attention with the shape's heads, half of every head rotated with stretched frequencies, capped
+    scores, chunks of 1,024 positions, a sink and a gate per head.  Parallel: on the left half the
+    shape's heads over a quarter of its key/value heads (the values are the keys), on the right the
+    delta rule with as many heads of the shape's head size as fill half the width, half as many q/k
+    heads, four taps.  A mixture of 32 experts, 4 a token, whose chosen experts together are as large
+    as the shape's feed-forward; the shape's vocabulary."""
+    width, hd, heads, kv = shape["hidden_size"], shape["head_dim"], shape["num_attention_heads"], shape["num_key_value_heads"]
+    mlp = {"kind": "moe", "expert": {"ff": max(64, shape["intermediate_size"] // 4 // 64 * 64)},
+           "router": {"experts": 32, "top": 4}}
+    attention = {"type": "attention", "mixer": {
+        "heads": heads, "kv_heads": kv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": 1024}, "softcap": 50.0,
+        "rot": {"dims": hd // 2, "base": 1000000.0, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}},
+        "mlp": mlp}
+    delta_heads = max(2, width // (2 * hd) // 2 * 2)
+    parallel = {"type": "parallel", "mixer": {
+        "left": {"heads": heads // 2, "kv_heads": max(1, kv // 4), "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+                 "rot": {"dims": hd // 2, "base": 500000.0}},
+        "left_scale": 1.0,
+        "right": {"heads": delta_heads, "kv_heads": delta_heads // 2, "dim": hd, "vdim": hd, "conv": 4},
+        "right_scale": 1.0}, "mlp": mlp}
+    return {"architecture": "Tukarax", "vocab": shape["vocab_size"], "width": width, "norm": {"eps": 1e-6},
+            "layers": [parallel if i % 2 == 0 else attention for i in range(layers)]}
+
+
 def design_steps(runner, vocab: int, batch: int, prompt_len: int, steps: int, warmup: int, seed: int) -> dict:
     """Milliseconds of one prompt step of ``prompt_len`` tokens (median of five), and of a
     decode step of ``batch`` requests behind such prompts (mean of ``steps``), through the step
@@ -396,7 +422,7 @@ def design_steps(runner, vocab: int, batch: int, prompt_len: int, steps: int, wa
 
 
 def design_main(args) -> int:
-    """``--design vupuzen|pavitar|gimudra``: prefill and decode of models of that design of random
+    """``--design vupuzen|pavitar|gimudra|tukarax``: prefill and decode of models of that design of random
     weights at the layer sizes of ``--shape`` (and of the other shapes named by ``--design-shapes``),
     beside the model of the design ``--beside`` (Qwen3 unless told otherwise) of the same sizes and
     number of layer runs, both through the same step function over pages of 256 tokens with decode
@@ -417,7 +443,8 @@ def design_main(args) -> int:
         shape = SHAPES[name]
         layers = args.layers or 8
         pages = (args.batch + 1) * (-(-(prompt_len + steps + warmup + 8) // PAGE_SIZE) + 1)
-        makers = {"vupuzen": vupuzen_json, "pavitar": pavitar_json, "gimudra": gimudra_json, "qwen3": config_json}
+        makers = {"vupuzen": vupuzen_json, "pavitar": pavitar_json, "gimudra": gimudra_json, "tukarax": tukarax_json,
+                  "qwen3": config_json}
         for design, raw in ((args.design, makers[args.design](shape, layers)), (beside, makers[beside](shape, layers))):
             config = PylonConfig(dtype=args.dtype, max_batch_size=args.batch + 1, max_queue_size=args.batch + 1,
                                  page_size=PAGE_SIZE, prefill_chunk_size=prompt_len, num_pages=pages,
@@ -468,9 +495,9 @@ def main() -> int:
     parser.add_argument("--no-peaks", action="store_true", help="skip the probes of this device's own peaks")
     parser.add_argument("--mixed", action="store_true",
                         help="also time a step of --batch decoded tokens beside a 2,048-token prompt portion")
-    parser.add_argument("--design", choices=("qwen3", "vupuzen", "pavitar", "gimudra"), default="qwen3",
-                        help="vupuzen, pavitar, gimudra: that design beside Qwen3 at equal sizes instead of the default workload")
-    parser.add_argument("--beside", choices=("qwen3", "vupuzen", "pavitar"), default="qwen3",
+    parser.add_argument("--design", choices=("qwen3", "vupuzen", "pavitar", "gimudra", "tukarax"), default="qwen3",
+                        help="vupuzen, pavitar, gimudra, tukarax: that design beside Qwen3 at equal sizes instead of the default workload")
+    parser.add_argument("--beside", choices=("qwen3", "vupuzen", "pavitar", "gimudra"), default="qwen3",
                         help="with another --design: the design it is measured beside (default qwen3)")
     parser.add_argument("--design-shapes", default="", help="with another --design: further shapes, with commas")
     parser.add_argument("--prefill-only", action="store_true",

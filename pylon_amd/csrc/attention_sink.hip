@@ -39,12 +39,22 @@ __device__ __forceinline__ uint32_t as_pack(float a, float b) {
 }
 
 // KS: steps of 32 key elements (dim <= 32 KS); NV: tiles of 16 value elements (vdim <= 16 NV).
+// scale * s, or with a cap c > 0: c * tanh(scale * s / c), the tangent as 1 - 2 / (e^(2x) + 1)
+// (it ends at 1 and -1 where the exponential overflows or vanishes).
+__device__ __forceinline__ float capped_score(float s, float scale, float cap) {
+  const float v = s * scale;
+  if (!(cap > 0.f)) return v;
+  const float e = __expf(2.0f * v / cap);
+  return cap * (1.0f - 2.0f / (e + 1.0f));
+}
+
 template <int KS, int NV>
 __global__ __launch_bounds__(512) void attention_sink_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, const int* __restrict__ positions, int n_heads, int n_kv_heads, int dim, int vdim, int page_size, float scale,
-    const float* __restrict__ bias, int bucket_len, int sink, int cuts, float* __restrict__ partial, int window) {
+    const float* __restrict__ bias, int bucket_len, int sink, int cuts, float* __restrict__ partial, int window,
+    float softcap, const float* __restrict__ sink_logit) {
   // eight waves: wave & 3 names the head of the group, wave >> 2 which 16 of the tile's 32 tokens, so
   // that every SIMD holds two waves that fill each other's waits
   constexpr int waves_per_group = 4;
@@ -108,8 +118,9 @@ __global__ __launch_bounds__(512) void attention_sink_kernel(
   float m_run[AS_QT], l_run[AS_QT];
 #pragma unroll
   for (int qt = 0; qt < AS_QT; ++qt) {
-    // the sink: a key of score 0 without a value (one lane of a query's four carries its one)
-    m_run[qt] = (sink && cut == 0) ? 0.f : -INFINITY;
+    // the sink: a key without a value (one lane of a query's four carries its one) whose score is 0,
+    // or the head's learned number
+    m_run[qt] = (sink && cut == 0) ? (sink_logit != nullptr ? sink_logit[head] : 0.f) : -INFINITY;
     l_run[qt] = (sink && cut == 0 && grp == 0) ? 1.f : 0.f;
 #pragma unroll
     for (int dt = 0; dt < NV; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -239,7 +250,7 @@ __global__ __launch_bounds__(512) void attention_sink_kernel(
           idx = idx < bucket_len - 1 ? idx : bucket_len - 1;
           bias = tbl[idx];
         }
-        const float v = fmaf(s[qt][e >> 2][e & 3], scale, bias);
+        const float v = capped_score(s[qt][e >> 2][e & 3], scale, softcap) + bias;
         sc[e] = (dist >= 0 && key >= qfirst[qt]) ? v : -INFINITY;
         top = fmaxf(top, sc[e]);
       }
@@ -335,7 +346,8 @@ __global__ __launch_bounds__(256) void attention_sink_decode_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ positions, int n_heads, int n_kv_heads, int dim, int vdim, int page_size, float scale,
-    const float* __restrict__ bias, int bucket_len, int sink, int cuts, float* __restrict__ partial, int window) {
+    const float* __restrict__ bias, int bucket_len, int sink, int cuts, float* __restrict__ partial, int window,
+    float softcap, const float* __restrict__ sink_logit) {
   extern __shared__ float bias_lds[];  // [group][bucket_len]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
@@ -373,7 +385,7 @@ __global__ __launch_bounds__(256) void attention_sink_decode_kernel(
 #pragma unroll
   for (int dt = 0; dt < NV; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   const bool first = sink && cut == 0 && wave == 0;  // the sink belongs to one partial result
-  float m_run = first ? 0.f : -INFINITY;
+  float m_run = first ? (sink_logit != nullptr ? sink_logit[my_head] : 0.f) : -INFINITY;
   float l_run = (first && grp == 0) ? 1.f : 0.f;
 
   const int first_key = first_visible(pos, window);  // a window, a chunk: the walk starts at its block
@@ -434,7 +446,7 @@ __global__ __launch_bounds__(256) void attention_sink_decode_kernel(
         idx = idx < bucket_len - 1 ? idx : bucket_len - 1;
         add = tbl[idx];
       }
-      const float v = fmaf(s[e >> 2][e & 3], scale, add);
+      const float v = capped_score(s[e >> 2][e & 3], scale, softcap) + add;
       sc[e] = (dist >= 0 && key >= first_key) ? v : -INFINITY;
       top = fmaxf(top, sc[e]);
     }
@@ -549,7 +561,8 @@ extern "C" int pylon_attention_sink(void* out, const void* q, long long q_stride
                                     const int* positions, int n_tiles, int n_heads, int n_kv_heads, int dim, int vdim, int page_size,
                                     float scale, const float* bias, int bucket_len, int sink,
                                     int cuts, float* partial, long long partial_floats, int tokens, int window,
-                                    hipStream_t stream) {
+                                    float softcap, const float* sink_logit, hipStream_t stream) {
+  PYLON_REQUIRE(sink_logit == nullptr || sink, "attention_sink: a learned sink is a sink");
   PYLON_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                 "attention_sink: %d query heads cannot be grouped over %d key/value heads", n_heads, n_kv_heads);
   PYLON_REQUIRE(dim >= 8 && dim % 8 == 0 && dim <= 256, "attention_sink: keys of a multiple of 8 up to 256 elements, got %d", dim);
@@ -588,7 +601,7 @@ extern "C" int pylon_attention_sink(void* out, const void* q, long long q_stride
     hipLaunchKernelGGL((attention_sink_decode_kernel<KS, NV>), dim3(static_cast<unsigned>(wgs)), dim3(256), lds_d,    \
                        stream, (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,           \
                        block_table, table_width, positions, n_heads, n_kv_heads, dim, vdim, page_size, scale, bias,  \
-                       bias != nullptr ? bucket_len : 1, sink, cuts, partial, window);                               \
+                       bias != nullptr ? bucket_len : 1, sink, cuts, partial, window, softcap, sink_logit);          \
   } while (0)
 #define PICK_D(KS)                  \
   do {                              \
@@ -628,7 +641,8 @@ extern "C" int pylon_attention_sink(void* out, const void* q, long long q_stride
                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
   hipLaunchKernelGGL((attention_sink_kernel<KS, NV>), grid, block, lds, stream, (bf16_t*)out, (const bf16_t*)q, \
                      q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, tiles, \
-                     positions, n_heads, n_kv_heads, dim, vdim, page_size, scale, bias, table_len, sink, cuts, partial, window); \
+                     positions, n_heads, n_kv_heads, dim, vdim, page_size, scale, bias, table_len, sink, cuts, partial, window, \
+                     softcap, sink_logit); \
   } while (0)
 #define PICK_NV(KS)                 \
   do {                              \

@@ -21,7 +21,7 @@ qkv_prepare_wide_kernel(T* __restrict__ q_out, T* __restrict__ k_cache, T* __res
                         const float* __restrict__ k_weight, float eps, const float* __restrict__ inv_freq,
                         int rot_dim, int interleaved, const int* __restrict__ positions,
                         const int* __restrict__ slot_map, int n_heads, int n_kv_heads, int head_dim, int v_dim,
-                        int store, int per_head, float rot_scale, int v_offset) {
+                        int store, int per_head, float rot_scale, int v_offset, int v_page) {
   extern __shared__ float turn[];  // cos then sin of the token's rot_dim/2 angles, then per head 1/rms
   float* head_inv = turn + (rot_dim > 0 ? rot_dim : 1);
   __shared__ float scratch[16];
@@ -107,9 +107,16 @@ qkv_prepare_wide_kernel(T* __restrict__ q_out, T* __restrict__ k_cache, T* __res
     }
   }
   if (store) {
-    T* dst = v_cache + static_cast<size_t>(slot_map[t]) * v_size;
     const T* src = row + v_offset;
-    for (int e = tid; e < v_size; e += QW_THREADS) dst[e] = src[e];
+    if (v_page > 0) {
+      // values transposed inside their page: [page, kv head, element, slot in page]
+      const int slot = slot_map[t];
+      T* dst = v_cache + static_cast<size_t>(slot / v_page) * v_size * v_page + slot % v_page;
+      for (int e = tid; e < v_size; e += QW_THREADS) dst[static_cast<size_t>(e) * v_page] = src[e];
+    } else {
+      T* dst = v_cache + static_cast<size_t>(slot_map[t]) * v_size;
+      for (int e = tid; e < v_size; e += QW_THREADS) dst[e] = src[e];
+    }
   }
 }
 
@@ -119,12 +126,13 @@ qkv_prepare_wide_kernel(T* __restrict__ q_out, T* __restrict__ k_cache, T* __res
 // [n_heads*head_dim] and k_weight [n_kv_heads*head_dim] float, or null for no norm.  inv_freq:
 // rot_dim/2 floats (rot_dim 0: no rotation); interleaved 1 pairs neighbours, 0 halves.
 // per_head 1: q_weight and k_weight hold head_dim floats and every head is normed by itself.
-// v_offset: where in a row the values start (with store).
+// v_offset: where in a row the values start (with store).  v_page > 0: the values' cache is
+// [pages, n_kv_heads, v_dim, v_page] (transposed inside pages of v_page slots).
 extern "C" int pylon_qkv_prepare_wide(void* q_out, void* k_cache, void* v_cache, const void* qkv, int dtype,
                                       long long row_stride, const float* q_weight, const float* k_weight, float eps,
                                       const float* inv_freq, int rot_dim, int interleaved, const int* positions,
                                       const int* slot_map, int tokens, int n_heads, int n_kv_heads, int head_dim,
-                                      int v_dim, int store, int per_head, float rot_scale, int v_offset,
+                                      int v_dim, int store, int per_head, float rot_scale, int v_offset, int v_page,
                                       hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(dtype), "qkv_prepare_wide: unknown dtype");
   PYLON_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && v_dim > 0,
@@ -150,11 +158,11 @@ extern "C" int pylon_qkv_prepare_wide(void* q_out, void* k_cache, void* v_cache,
     hipLaunchKernelGGL((qkv_prepare_wide_kernel<float>), dim3(tokens), dim3(QW_THREADS), lds, stream, (float*)q_out,
                        (float*)k_cache, (float*)v_cache, (const float*)qkv, row_stride, q_weight, k_weight, eps,
                        inv_freq, rot_dim, interleaved, positions, slot_map, n_heads, n_kv_heads, head_dim, v_dim,
-                       store, per_head, rot_scale, v_offset);
+                       store, per_head, rot_scale, v_offset, v_page);
   else
     hipLaunchKernelGGL((qkv_prepare_wide_kernel<bf16_t>), dim3(tokens), dim3(QW_THREADS), lds, stream,
                        (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, (const bf16_t*)qkv, row_stride, q_weight,
                        k_weight, eps, inv_freq, rot_dim, interleaved, positions, slot_map, n_heads, n_kv_heads,
-                       head_dim, v_dim, store, per_head, rot_scale, v_offset);
+                       head_dim, v_dim, store, per_head, rot_scale, v_offset, v_page);
   PYLON_LAUNCHED("qkv_prepare_wide");
 }

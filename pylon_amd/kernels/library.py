@@ -32,7 +32,7 @@ _SIGNATURES = {
     "pylon_silu_gate": [P, I, P, I, I, I, P],
     "pylon_qkv_prepare": [P, P, P, P, I, L, P, P, F, P, I, P, P, I, I, I, I, I, P],
     "pylon_paged_attention": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, I, L, P, P, I, I, I, F, P, P],
-    "pylon_attention_sink": [P, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, P, I, I, I, P, L, I, I, P],
+    "pylon_attention_sink": [P, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, P, I, I, I, P, L, I, I, F, P, P],
     "pylon_add_normed_rmsnorm": [P, I, P, P, I, I, L, P, F, P, I, P, I, I, F, P, P, P],
     "pylon_depth_mix": [P, I, P, P, I, I, L, P, P, P, L, I, P, P, I, I, F, P],
     "pylon_short_conv": [P, I, P, I, P, I, P, P, P, I, I, I, I, L, I, P],
@@ -56,7 +56,7 @@ _SIGNATURES = {
     "pylon_argmax_static": [P, P, I, I, L, P, P, P],
     "pylon_probe_read": [P, L, P, P],
     "pylon_sample": [P, P, I, I, L, P, P, P, P, P, P],
-    "pylon_qkv_prepare_wide": [P, P, P, P, I, L, P, P, F, P, I, I, P, P, I, I, I, I, I, I, I, F, I, P],
+    "pylon_qkv_prepare_wide": [P, P, P, P, I, L, P, P, F, P, I, I, P, P, I, I, I, I, I, I, I, F, I, I, P],
     "pylon_latent_prepare": [P, P, P, P, L, I, P, P, F, P, I, I, I, I, I, P],
     "pylon_head_project": [P, P, I, L, P, I, P, I, I, I, I, P],
     "pylon_gate_heads": [P, I, P, L, I, P],
@@ -69,7 +69,7 @@ _SIGNATURES = {
     "pylon_grouped_down": [P, P, L, P, L, P, I, I, I, I, P],
     "pylon_sigmoid_gate": [P, I, P, L, L, I, I, P],
     "pylon_scaled_sum": [P, P, I, I, F, P, I, I, F, L, P],
-    "pylon_delta_rule": [P, I, L, P, L, I, I, I, P, L, I, I, I, P, P, P, P, P, P, I, I, I, I, I, F, F, F, P],
+    "pylon_delta_rule": [P, I, L, P, L, I, I, I, P, L, I, I, I, P, P, P, P, P, P, I, I, I, I, I, F, F, F, I, P, I, P],
     "pylon_expert_combine": [P, P, P, P, P, P, I, I, I, P, P, L, P, P],
 }
 

@@ -309,7 +309,8 @@ def bias_by_distance(rel: torch.Tensor, bucket: torch.Tensor) -> torch.Tensor:
 def attention_sink(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                    tiles: Optional[torch.Tensor], positions: Optional[torch.Tensor], *, page_size: int, scale: float,
                    bias: Optional[torch.Tensor], sink: bool, cuts: int = 1, window: Optional[int] = None,
-                   chunk: Optional[int] = None) -> torch.Tensor:
+                   chunk: Optional[int] = None, softcap: Optional[float] = None,
+                   sink_logit: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention with a bias by distance and a sink on the matrix cores: bfloat16 ``q``
     ``[tokens, heads, head_dim]`` (maybe a slice of wider rows), keys ``[pages, page_size, kv_heads,
     head_dim]``, values transposed inside their pages ``[pages, kv_heads, v_dim, page_size]``.
@@ -317,9 +318,15 @@ def attention_sink(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     ``tiles`` int32 ``[n, 4]`` (first token, count <= 32, block-table row, first position); or None
     with ``positions``: every token a tile of its own on its own row of the table.  ``cuts``
     workgroups share the keys of a tile and a second kernel merges their float partial results.
-    ``window`` / ``chunk``: which earlier keys a token sees (:func:`mask_code`)."""
+    ``window`` / ``chunk``: which earlier keys a token sees (:func:`mask_code`).  ``softcap``: the
+    scaled score ``s`` becomes ``softcap * tanh(s / softcap)`` before the bias; ``sink_logit`` (float32
+    ``[heads]``, with ``sink``): the sink's score per head in place of 0."""
     if q.dim() != 3 or k_cache.dim() != 4 or v_cache.dim() != 4:
         raise KernelError("attention_sink takes q [tokens, heads, head_dim] and 4-D caches")
+    if sink_logit is not None and (not sink or sink_logit.shape != (q.shape[1],)):
+        raise KernelError("attention_sink: sink_logit is float32 [heads] and goes with sink")
+    if softcap is not None and not softcap > 0:
+        raise KernelError("attention_sink: a soft cap is positive")
     tokens, n_heads, head_dim = q.shape
     pages, psize, n_kv_heads, hd = k_cache.shape
     v_dim = v_cache.shape[2]
@@ -353,7 +360,8 @@ def attention_sink(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
               block_table.shape[1], _dev(tiles, "tiles", torch.int32), _dev(positions, "positions", torch.int32),
               n_tiles, n_heads, n_kv_heads, head_dim, v_dim, page_size, float(scale), _dev(bias, "bias", torch.float32),
               0 if bias is None else bias.shape[1], 1 if sink else 0, int(cuts), _dev(partial, "partial"),
-              0 if partial is None else partial.numel(), tokens, mask_code(window, chunk), _stream())
+              0 if partial is None else partial.numel(), tokens, mask_code(window, chunk), float(softcap or 0.0),
+              _dev(sink_logit, "sink_logit", torch.float32), _stream())
     return out
 
 
@@ -682,10 +690,27 @@ def delta_rule_ok(dim: int, vdim: int) -> bool:
     return dim >= 1 and vdim >= 1 and r <= 128 and vdim * p <= 1024 and (r <= 64 or vdim * p <= 256)
 
 
+def delta_rule_col_groups(rows: int, heads: int, dim: int, vdim: int, max_count: Optional[int],
+                          units: Optional[int] = None) -> int:
+    """Over how many workgroups the columns of a head's state are dealt: one for steps of short rows
+    (one launch, the norm inside); for rows of 64 tokens and more a power of two of at most 16 that
+    divides ``vdim``, leaves every workgroup at least 8 columns and does not start more workgroups
+    than twice the compute units."""
+    if max_count is None or max_count < 64:
+        return 1
+    units = units or _lib.compute_units()
+    groups = 1
+    while (groups < 16 and vdim % (groups * 2) == 0 and vdim // (groups * 2) >= 8
+           and rows * heads * groups * 2 <= 2 * units and delta_rule_ok(dim, vdim // (groups * 2))):
+        groups *= 2
+    return groups
+
+
 def delta_rule(qkv: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, a_log: torch.Tensor,
                dt_bias: torch.Tensor, norm_weight: torch.Tensor, row_start: torch.Tensor, row_slots: torch.Tensor, *,
                rows: int, heads: int, kv_heads: int, dim: int, vdim: int, gate_off: int, beta_off: int,
-               decay_off: int, eps: float, unit_eps: float, q_scale: float, out_dtype: torch.dtype) -> torch.Tensor:
+               decay_off: int, eps: float, unit_eps: float, q_scale: float, out_dtype: torch.dtype,
+               max_count: Optional[int] = None, col_groups: Optional[int] = None) -> torch.Tensor:
     """The gated delta rule over the rows of a step: per request and head ``S <- g S; u = beta (v -
     S^T k); S <- S + k u^T; o = S^T q``.  ``qkv`` float32 ``[tokens, 2 kv_heads dim + heads vdim]``
     holds q, k and v (after their convolution and activation); q and k become unit vectors per head
@@ -694,7 +719,9 @@ def delta_rule(qkv: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, a_log
     ``beta_off``) and of the decay (from ``decay_off``): ``beta = sigmoid(b)``, ``g = exp(-exp(a_log) *
     softplus(a + dt_bias))``.  ``state`` float32 ``[slots, heads, vdim, dim]`` (the state transposed)
     is read and left up to date.  Returns ``o / rms(o) * norm_weight * silu(gate)`` as ``[tokens,
-    heads * vdim]``."""
+    heads * vdim]``.  ``max_count`` (the most tokens a row brings) lets long rows have the columns of
+    a head's state dealt to several workgroups (:func:`delta_rule_col_groups`; ``col_groups`` says
+    it outright); the results are the same numbers either way."""
     if qkv.dim() != 2 or proj.dim() != 2 or qkv.dtype != torch.float32 or proj.dtype != torch.float32 \
             or qkv.stride(1) != 1 or proj.stride(1) != 1 or qkv.shape[0] != proj.shape[0]:
         raise KernelError("delta_rule takes float32 rows of q, k, v and of the projection, one per token")
@@ -715,13 +742,19 @@ def delta_rule(qkv: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, a_log
     if not qkv.is_cuda:
         raise KernelError("qkv must live on the GPU; there is no CPU path")
     out = torch.empty((tokens, heads * vdim), dtype=out_dtype, device=qkv.device)
+    if col_groups is None:
+        col_groups = delta_rule_col_groups(rows, heads, dim, vdim, max_count)
+    if col_groups < 1 or vdim % col_groups or not delta_rule_ok(dim, vdim // col_groups):
+        raise KernelError(f"delta_rule: {vdim} columns cannot be dealt to {col_groups} workgroups")
+    raw = torch.empty((tokens, heads * vdim), dtype=torch.float32, device=qkv.device) if col_groups > 1 else None
     _lib.call("pylon_delta_rule", _dev(out, "out"), dtype_code(out_dtype), heads * vdim, qkv.data_ptr(),
               qkv.stride(0) if tokens > 1 else qkv.shape[1], 0, qk, 2 * qk, proj.data_ptr(),
               proj.stride(0) if tokens > 1 else proj.shape[1], int(gate_off), int(beta_off), int(decay_off),
               _dev(a_log, "a_log", torch.float32), _dev(dt_bias, "dt_bias", torch.float32),
               _dev(norm_weight, "norm_weight", torch.float32), _dev(state, "state", torch.float32),
               _dev(row_start, "row_start", torch.int32), _dev(row_slots, "row_slots", torch.int32), rows, heads,
-              kv_heads, dim, vdim, float(eps), float(unit_eps), float(q_scale), _stream())
+              kv_heads, dim, vdim, float(eps), float(unit_eps), float(q_scale), int(col_groups), _dev(raw, "raw"),
+              tokens, _stream())
     return out
 
 
@@ -1252,7 +1285,8 @@ def qkv_prepare_wide(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: Optional[t
                      q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
                      inv_freq: Optional[torch.Tensor], rot_dim: int, interleaved: bool,
                      positions: Optional[torch.Tensor], slot_map: Optional[torch.Tensor], store_kv: bool,
-                     per_head: bool = False, rot_scale: float = 1.0, values_from_keys: bool = False) -> None:
+                     per_head: bool = False, rot_scale: float = 1.0, values_from_keys: bool = False,
+                     v_transposed: bool = False) -> None:
     """q/k/v preparation with norms over whole projections: ``q_weight`` (float32, all heads of q
     side by side) and ``k_weight`` norm the whole q row and the whole k row of a token (None: no
     norm); the first ``rot_dim`` elements of every head of q and k are rotated by ``position *
@@ -1261,7 +1295,9 @@ def qkv_prepare_wide(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: Optional[t
     by head with weights of ``head_dim`` elements.  ``rot_scale`` multiplies every cosine and
     sine.  ``values_from_keys``: there are no value columns; the values are the keys as projected,
     before norm and rotation (``v_dim`` is then ``head_dim``).  The rows of ``qkv`` may be wider
-    than q, k and v together (further columns of a fused projection are left alone)."""
+    than q, k and v together (further columns of a fused projection are left alone).
+    ``v_transposed``: the values go into their pages as ``[pages, kv_heads, v_dim, page_size]``
+    (``v_cache`` is given in that shape; the page's size is the keys' cache's)."""
     if qkv.dim() != 2 or qkv.stride(1) != 1:
         raise KernelError("qkv_prepare_wide takes a 2-D projection output with contiguous rows")
     tokens, width = qkv.shape
@@ -1285,8 +1321,11 @@ def qkv_prepare_wide(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: Optional[t
             raise KernelError("qkv_prepare_wide: storing needs k_cache, v_cache and one slot per token")
         if k_cache.dtype != qkv.dtype or k_cache.shape[-2:] != (n_kv_heads, head_dim):
             raise KernelError(f"qkv_prepare_wide: k_cache must be [..., {n_kv_heads}, {head_dim}] of {qkv.dtype}")
-        if v_cache.dtype != qkv.dtype or v_cache.shape[-2:] != (n_kv_heads, v_dim):
-            raise KernelError(f"qkv_prepare_wide: v_cache must be [..., {n_kv_heads}, {v_dim}] of {qkv.dtype}")
+        v_tail = tuple(v_cache.shape[-3:-1]) if v_transposed else tuple(v_cache.shape[-2:])
+        if v_cache.dtype != qkv.dtype or v_tail != (n_kv_heads, v_dim) or \
+                (v_transposed and (k_cache.dim() != 4 or v_cache.shape[-1] != k_cache.shape[1])):
+            raise KernelError(f"qkv_prepare_wide: v_cache must be [..., {n_kv_heads}, {v_dim}] of {qkv.dtype} "
+                              "(or, transposed, [pages, kv_heads, v_dim, page_size])")
     if not qkv.is_cuda:
         raise KernelError("qkv must live on the GPU; there is no CPU path")
     _lib.call("pylon_qkv_prepare_wide", _dev(q_out, "q_out"), _dev(k_cache if store_kv else None, "k_cache"),
@@ -1295,7 +1334,7 @@ def qkv_prepare_wide(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: Optional[t
               _dev(inv_freq, "inv_freq", torch.float32), int(rot_dim), 1 if interleaved else 0,
               _dev(positions, "positions", torch.int32), _dev(slot_map if store_kv else None, "slot_map", torch.int32),
               tokens, n_heads, n_kv_heads, head_dim, v_dim, 1 if store_kv else 0, 1 if per_head else 0,
-              float(rot_scale), int(v_offset), _stream())
+              float(rot_scale), int(v_offset), int(k_cache.shape[1]) if (store_kv and v_transposed) else 0, _stream())
 
 
 def latent_prepare(down: torch.Tensor, cache: Optional[torch.Tensor], slot_map: Optional[torch.Tensor], *,

@@ -18,7 +18,10 @@ whose cosines and sines carry a factor (the position part's ``rot_scale``); scor
 ``softcap * tanh(s / softcap)``; a learned sink per head in the softmax's denominator; values that
 are the keys as projected (``values_from_keys``: no value projection); and an output gate
 ``sigmoid(W_g h)`` per head or per element on the heads' outputs, whose rows are the last of the
-fused projection ``[q; k; v; g]``.  Capped scores and the learned sink run on the general kernel.
+fused projection ``[q; k; v; g]``.  Capped scores and the learned sink run, for bfloat16 over pages
+of a multiple of 32 tokens, on the matrix-core kernel that :class:`SinkAttention` uses (prompt tiles and
+single tokens with their keys cut over workgroups; the values then lie transposed inside their pages),
+and otherwise on the general kernel.
 """
 from __future__ import annotations
 
@@ -99,7 +102,19 @@ class Attention(Part):
         a request are shared between workgroups and waves."""
         limit = self.spec.window if self.spec.window is not None else self.spec.chunk
         span = bound if limit is None else min(bound, limit)
+        if self.special:
+            if self.dtype != torch.bfloat16:
+                return ("attention", "general")
+            return ("attention", "sink", ops.sink_cuts(rows, self.spec.n_heads, self.spec.n_kv_heads, span))
         return ("attention",) + tuple(ops.decode_launch(rows, self.spec.n_kv_heads, span))
+
+    def _sink_kernel(self, page_size: int) -> bool:
+        """Whether capped scores and the sink run on the matrix cores (the values then lie transposed
+        inside their pages: a property of the model's type, the heads' sizes and the page's, so every
+        step of a runner stores and reads them one way)."""
+        spec = self.spec
+        return self.special and ops.attention_sink_ok(self.dtype, head_dim=spec.head_dim, v_dim=spec.value_dim,
+                                                      page_size=page_size, bucket_len=0)
 
     def forward(self, h: torch.Tensor, ctx, cache, stores: bool) -> torch.Tensor:
         spec = self.spec
@@ -127,7 +142,11 @@ class Attention(Part):
                                            out_dtype=self.dtype)
         qkv = ops.linear(h, weight, out_dtype=self.dtype)
         q = torch.empty((tokens, spec.n_heads, spec.head_dim), dtype=self.dtype, device=h.device)
-        if self.plain:
+        on_cores = self._sink_kernel(cache.page_size) if cache.k is not None else False
+        v_cache = cache.v
+        if on_cores:
+            v_cache = cache.v.view(cache.v.shape[0], spec.n_kv_heads, spec.value_dim, cache.page_size)
+        if self.plain and not on_cores:
             ops.qkv_prepare(
                 qkv, q, cache.k, cache.v,
                 n_heads=spec.n_heads, n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim,
@@ -139,7 +158,7 @@ class Attention(Part):
         else:
             # norms over whole projections, neighbours rotated together, values of another size
             ops.qkv_prepare_wide(
-                qkv, q, cache.k, cache.v,
+                qkv, q, cache.k, v_cache,
                 n_heads=spec.n_heads, n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim, v_dim=spec.value_dim,
                 q_weight=self.params.get("q_norm"), k_weight=self.params.get("k_norm"), eps=spec.qk_norm_eps,
                 inv_freq=rotary[0] if rotary else None, rot_dim=rotary[1] if rotary else 0,
@@ -147,10 +166,17 @@ class Attention(Part):
                 positions=ctx.positions, slot_map=cache.slot_map, store_kv=stores,
                 per_head=spec.qk_norm and spec.qk_norm_over == "head",
                 rot_scale=getattr(self.position, "rot_scale", 1.0), values_from_keys=spec.values_from_keys,
+                v_transposed=on_cores,
             )
         # the matrix-core kernels take values as large as keys, plain scores and no sink
         same_size = spec.value_dim == spec.head_dim and not self.special
-        if same_size and ctx.decode_only and ops.decode_attention_ok(q, cache.k):
+        if on_cores:
+            tiles = None if ctx.decode_only else ctx.token_tiles(ops.SINK_TILE)
+            cuts = ops.sink_cuts(tokens, spec.n_heads, spec.n_kv_heads, self._span(ctx)) if ctx.decode_only else 1
+            context = ops.attention_sink(q, cache.k, v_cache, cache.block_table, tiles, ctx.positions,
+                                         page_size=cache.page_size, scale=spec.scale, bias=None, sink=spec.sink,
+                                         cuts=cuts, softcap=spec.softcap, sink_logit=self.params.get("sink"), **mask)
+        elif same_size and ctx.decode_only and ops.decode_attention_ok(q, cache.k):
             cuts, splits = ops.decode_launch(tokens, spec.n_kv_heads, self._span(ctx))
             # in a decode-only step token t is row t
             context = ops.attention_decode(

@@ -70,7 +70,7 @@ class GatedDeltaRule(Part):
             ctx.row_start, ctx.row_slots, rows=ctx.rows, heads=spec.n_heads, kv_heads=spec.n_kv_heads,
             dim=spec.head_dim, vdim=spec.v_head_dim, gate_off=self.gate_off, beta_off=self.beta_off,
             decay_off=self.decay_off, eps=spec.norm_eps, unit_eps=spec.unit_eps, q_scale=spec.head_dim ** -0.5,
-            out_dtype=self.dtype)
+            out_dtype=self.dtype, max_count=ctx.max_count)
         return ops.linear_for_residual(mixed, self.params["out"], out_dtype=self.dtype)
 
 

@@ -98,6 +98,8 @@ def test_delta_rule_in_portions_of_two_requests_over_reused_slots(ops, heads, kv
     for slot in slots.values():
         state[slot].zero_()  # what the manager does when it hands a slot out
     plan = [{"x": 5}, {"x": 1, "y": 2}, {"y": 1}, {"x": 18, "y": 1}, {"x": 1}, {"y": 19, "x": 16}]
+    # a head's columns dealt to several workgroups where they divide (the norm then in a second kernel)
+    groups = max([g for g in (2, 4, 8, 16) if vdim % g == 0 and vdim // g >= 4] + [1])
     pos = {rid: 0 for rid in lengths}
     got = {rid: [] for rid in lengths}
     pad = 3  # the projection's rows are wider than what the kernel reads
@@ -114,7 +116,8 @@ def test_delta_rule_in_portions_of_two_requests_over_reused_slots(ops, heads, kv
         out = ops.delta_rule(dev(np.concatenate(qkv_rows)), dev(np.concatenate(proj_rows)), state, dev(a_log), dev(dt_bias),
                              dev(norm_w), i32(starts), i32(slots[r] for r in rows), rows=len(rows), heads=heads,
                              kv_heads=kv_heads, dim=dim, vdim=vdim, gate_off=pad, beta_off=pad + vv,
-                             decay_off=pad + vv + heads, eps=eps, unit_eps=1e-6, q_scale=dim ** -0.5, out_dtype=out_dtype)
+                             decay_off=pad + vv + heads, eps=eps, unit_eps=1e-6, q_scale=dim ** -0.5, out_dtype=out_dtype,
+                             col_groups=groups if len(step) % 2 else 1)  # the two ways in turns over one state
         out = out.float().cpu().numpy()
         for i, rid in enumerate(rows):
             got[rid].append(out[starts[i]: starts[i + 1]])
@@ -278,6 +281,21 @@ def test_attention_with_a_cap_and_a_sink_at_the_edges_of_chunks_and_pages(ops, s
         out = ops.paged_attention(dev(q[first:], dtype), k_cache, v_cache, table, i32([0] * (n - first)), i32(range(first, n)),
                                   page_size=page, window=None, chunk=size, scale=scale, softcap=cap, sink_logit=dev(sink))
         close(out.float().cpu().numpy(), want[first:], bound, f"from {first}")
+    if dtype == torch.bfloat16:
+        # the matrix-core kernel over the same pages, the values transposed inside them: prompt tiles of up
+        # to 32 tokens from position 0 and from 143, then every position as a single token with its keys
+        # in one piece and cut over 2 and 8 workgroups
+        v_t = v_cache.view(pool, page, groups, vdim).permute(0, 2, 3, 1).contiguous()
+        for first in (0, 143):
+            tiles = i32(x for a in range(first, n, 32) for x in (a - first, min(32, n - a), 0, a)).view(-1, 4)
+            out = ops.attention_sink(dev(q[first:], dtype), k_cache, v_t, table, tiles, None, page_size=page, scale=scale,
+                                     bias=None, sink=True, chunk=size, softcap=cap, sink_logit=dev(sink))
+            close(out.float().cpu().numpy(), want[first:], bound, f"matrix cores from {first}")
+        for cuts in (1, 2, 8):
+            out = ops.attention_sink(dev(q, dtype), k_cache, v_t, table.expand(n, -1).contiguous(), None, i32(range(n)),
+                                     page_size=page, scale=scale, bias=None, sink=True, cuts=cuts, chunk=size,
+                                     softcap=cap, sink_logit=dev(sink))
+            close(out.float().cpu().numpy(), want, bound, f"single tokens, {cuts} cuts")
     # the cap and the sink matter in this case: without either the result is another
     bare = plain.softmax_attention(q, k, v, scale, plain.visible(n, size), None, sink)
     assert np.abs(bare - want).max() > 0.05
