@@ -12,7 +12,8 @@
 // thread (j, p) keeps a slice of R elements of column j of S (P slices a column, the P threads of
 // a column side by side in one wave, so the two sums over dim end in a few lane exchanges).  The
 // row's tokens go by in pieces of up to CT: the waves first prepare a piece (a wave a token: unit
-// vectors, beta, decay and the values into LDS), then every thread walks the piece token by token
+// vectors, beta, decay and the values into LDS; in the code: a few threads a token, all tokens of the
+// piece at once, the next piece's rows already on their way), then every thread walks the piece token by token
 // with no barrier in between, then the waves norm and gate the piece's outputs.  The state is
 // read from the request's slot at the start and written back at the end; it is kept transposed,
 // [slot, head, vdim, dim], so that a thread's slice is contiguous.
@@ -24,16 +25,19 @@
 // then leave o unnormed in a float buffer, and a second small kernel norms and gates it.
 #include "common.h"
 
-#define DR_PAD 4  // floats between two slices of q or k in LDS (keeps the slices' reads off one bank)
+#define DR_PAD 4   // floats between two slices of q or k in LDS (keeps the slices' reads off one bank)
+#define DR_HOLD 8  // elements of q, of k and of v that a thread may hold of the next piece
 
-template <int RT, int MAXT, typename TO>
+#define DR_C 16  // tokens of a piece in the chunked form
+
+template <int RT, int MAXT, bool CHUNK, typename TO>
 __global__ void __launch_bounds__(MAXT)
 delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __restrict__ qkv, long long qkv_stride,
                   int q_off, int k_off, int v_off, const float* __restrict__ proj, long long proj_stride, int g_off,
                   int b_off, int a_off, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
                   const float* __restrict__ norm_w, float* __restrict__ state, const int* __restrict__ row_start,
                   const int* __restrict__ row_slots, int heads, int kv_heads, int dim, int vdim, int P, int R, int CT,
-                  float eps, float unit_eps, float q_scale, int col_groups, float* __restrict__ raw) {
+                  float eps, float unit_eps, float q_scale, int col_groups, float* __restrict__ raw, int TPT) {
   extern __shared__ __attribute__((aligned(16))) float dr_lds[];
   const int cg = blockIdx.x % col_groups, rh = blockIdx.x / col_groups;
   const int row = rh / heads, h = rh - row * heads;
@@ -51,7 +55,13 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
   float* vs = ks + CT * KS;         // [CT][vg]
   float* os = vs + CT * vg;         // [CT][vg]
   float* betas = os + CT * vg;      // [CT]
-  float* decays = betas + CT;       // [CT]
+  float* decays = betas + CT;       // [CT]; in the chunked form the decays' logarithms
+  // chunked form only: A[t][s] = (G_t / G_s) k_s.k_t, B[t][s] = (G_t / G_s) k_s.q_t with G_t the product of
+  // the piece's decays up to token t; G itself; G_last / G_s
+  float* amat = decays + CT;        // [DR_C][DR_C]
+  float* bmat = amat + DR_C * DR_C; // [DR_C][DR_C]
+  float* gcum = bmat + DR_C * DR_C; // [DR_C]
+  float* gend = gcum + DR_C;        // [DR_C]
 
   float S[RT];
   float* st = state + ((static_cast<size_t>(row_slots[row]) * heads + h) * vdim + j0 + (owner ? j : 0)) * dim + p * R;
@@ -59,65 +69,247 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
   for (int r = 0; r < RT; ++r) S[r] = (owner && r < R && p * R + r < dim) ? st[r] : 0.f;
 
   const float rate = expf(a_log[h]), shift = dt_bias[h];
+  // A piece's rows are prepared by TPT threads a token, all tokens of the piece at once.  Where a
+  // thread's share is at most DR_HOLD elements of q, of k and of v, the next piece's rows are fetched
+  // into registers before the walk over this piece, so that their way from memory is hidden behind it.
+  const int ti = tid / TPT, sub = tid - ti * TPT;
+  const bool held = dim <= DR_HOLD * TPT && vg <= DR_HOLD * TPT;
+  float rq[DR_HOLD], rk[DR_HOLD], rv[DR_HOLD], rb = 0.f, ra = 0.f;
+  auto fetch = [&](int c0) {
+    const int n = end - c0 < CT ? end - c0 : CT;
+    if (ti >= n) return;
+    const size_t t = static_cast<size_t>(c0 + ti);
+    const float* qrow = qkv + t * qkv_stride + q_off + hk * dim;
+    const float* krow = qkv + t * qkv_stride + k_off + hk * dim;
+    const float* vrow = qkv + t * qkv_stride + v_off + h * vdim + j0;
+#pragma unroll
+    for (int e = 0; e < DR_HOLD; ++e) {
+      const int d = sub + e * TPT;
+      rq[e] = d < dim ? qrow[d] : 0.f;
+      rk[e] = d < dim ? krow[d] : 0.f;
+      rv[e] = d < vg ? vrow[d] : 0.f;
+    }
+    if (sub == 0) {
+      rb = proj[t * proj_stride + b_off + h];
+      ra = proj[t * proj_stride + a_off + h];
+    }
+  };
+  // the slices' pads (and the elements past dim) stay zero: only real elements are ever written
+  for (int e = tid; e < 2 * CT * KS; e += blockDim.x) qs[e] = 0.f;
+  if (held) fetch(begin);
+  __syncthreads();
   for (int c0 = begin; c0 < end; c0 += CT) {
     const int n = end - c0 < CT ? end - c0 : CT;
-    // a wave a token: unit q and k in the slices' layout (zeros where a slice has no element)
-    for (int i = wave; i < n; i += nwaves) {
-      const size_t t = static_cast<size_t>(c0 + i);
+    if (ti < n) {
+      const size_t t = static_cast<size_t>(c0 + ti);
       const float* qrow = qkv + t * qkv_stride + q_off + hk * dim;
       const float* krow = qkv + t * qkv_stride + k_off + hk * dim;
       const float* vrow = qkv + t * qkv_stride + v_off + h * vdim + j0;
       float sq = 0.f, sk = 0.f;
-      for (int d = lane; d < dim; d += PYLON_WAVE) {
-        sq = fmaf(qrow[d], qrow[d], sq);
-        sk = fmaf(krow[d], krow[d], sk);
+      if (held) {
+#pragma unroll
+        for (int e = 0; e < DR_HOLD; ++e) {
+          sq = fmaf(rq[e], rq[e], sq);
+          sk = fmaf(rk[e], rk[e], sk);
+        }
+      } else {
+        for (int d = sub; d < dim; d += TPT) {
+          sq = fmaf(qrow[d], qrow[d], sq);
+          sk = fmaf(krow[d], krow[d], sk);
+        }
       }
-      const float iq = q_scale / sqrtf(wave_sum(sq) + unit_eps);
-      const float ik = 1.0f / sqrtf(wave_sum(sk) + unit_eps);
-      for (int e = lane; e < KS; e += PYLON_WAVE) {
-        const int pp = e / (RT + DR_PAD), r = e - pp * (RT + DR_PAD);
-        const int d = pp * R + r;
-        const bool there = r < R && d < dim;
-        qs[i * KS + e] = there ? qrow[d] * iq : 0.f;
-        ks[i * KS + e] = there ? krow[d] * ik : 0.f;
+      for (int off = TPT >> 1; off > 0; off >>= 1) {  // the TPT threads of a token lie side by side in one wave
+        sq += __shfl_xor(sq, off, PYLON_WAVE);
+        sk += __shfl_xor(sk, off, PYLON_WAVE);
       }
-      for (int d = lane; d < vg; d += PYLON_WAVE) vs[i * vg + d] = vrow[d];
-      if (lane == 0) {
-        const float* pr = proj + t * proj_stride;
-        betas[i] = 1.0f / (1.0f + expf(-pr[b_off + h]));
-        const float a = pr[a_off + h] + shift;
+      const float iq = q_scale / sqrtf(sq + unit_eps);
+      const float ik = 1.0f / sqrtf(sk + unit_eps);
+      if (held) {
+#pragma unroll
+        for (int e = 0; e < DR_HOLD; ++e) {
+          const int d = sub + e * TPT;
+          if (d < dim) {
+            const int at = ti * KS + (d / R) * (RT + DR_PAD) + d % R;
+            qs[at] = rq[e] * iq;
+            ks[at] = rk[e] * ik;
+          }
+          if (d < vg) vs[ti * vg + d] = rv[e];
+        }
+      } else {
+        for (int d = sub; d < dim; d += TPT) {
+          const int at = ti * KS + (d / R) * (RT + DR_PAD) + d % R;
+          qs[at] = qrow[d] * iq;
+          ks[at] = krow[d] * ik;
+        }
+        for (int d = sub; d < vg; d += TPT) vs[ti * vg + d] = vrow[d];
+        if (sub == 0) {
+          rb = proj[t * proj_stride + b_off + h];
+          ra = proj[t * proj_stride + a_off + h];
+        }
+      }
+      if (sub == 0) {
+        betas[ti] = 1.0f / (1.0f + expf(-rb));
+        const float a = ra + shift;
         const float soft = a > 20.f ? a : log1pf(expf(a));
-        decays[i] = expf(-rate * soft);
+        decays[ti] = CHUNK ? -rate * soft : expf(-rate * soft);
       }
     }
     __syncthreads();
+    if (held && c0 + CT < end) fetch(c0 + CT);  // on their way while this piece is walked
+    if constexpr (CHUNK) {
+      // The piece at once.  With G_t = g_1 ... g_t (the piece's decays) and S_0 the state before it:
+      //   u_t = beta_t (v_t - G_t S_0^T k_t - sum_{s<t} A[t][s] u_s),
+      //   o_t = G_t S_0^T q_t + sum_{s<=t} B[t][s] u_s,   S_n = G_n S_0 + sum_s (G_n / G_s) k_s u_s^T,
+      // which is the token-by-token rule written out.  The products with S_0 and the sums over the
+      // lanes of a column are independent over the piece's tokens, so their waits overlap; what is
+      // left in order is a short chain of multiply-adds in registers.
+      for (int idx = tid; idx < 2 * DR_C * DR_C; idx += blockDim.x) {
+        const int which = idx / (DR_C * DR_C), ts = idx - which * DR_C * DR_C;
+        const int t = ts / DR_C, sx = ts - t * DR_C;
+        float value = 0.f;
+        if (t < n && sx <= t) {
+          const float4* a4 = reinterpret_cast<const float4*>(ks + sx * KS);
+          const float4* b4 = reinterpret_cast<const float4*>((which ? qs : ks) + t * KS);
+          float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+#pragma unroll 8
+          for (int e = 0; e < KS / 4; ++e) {  // the pads hold zeros; several reads of LDS in flight
+            const float4 x = a4[e], y = b4[e];
+            d0 = fmaf(x.x, y.x, d0);
+            d1 = fmaf(x.y, y.y, d1);
+            d2 = fmaf(x.z, y.z, d2);
+            d3 = fmaf(x.w, y.w, d3);
+          }
+          d0 = (d0 + d1) + (d2 + d3);
+          d1 = 0.f;
+          float lg = 0.f;
+          for (int r = sx + 1; r <= t; ++r) lg += decays[r];
+          value = (d0 + d1) * expf(lg);
+        }
+        (which ? bmat : amat)[ts] = value;
+      }
+      if (tid < DR_C) {
+        float lg = 0.f, all = 0.f;
+        for (int r = 0; r < n; ++r) {
+          all += decays[r];
+          if (r <= tid) lg = all;
+        }
+        gcum[tid] = expf(lg);
+        gend[tid] = expf(all - lg);
+      }
+      __syncthreads();
+      if (owner) {
+        const float* kbase = ks + p * (RT + DR_PAD);
+        const float* qbase = qs + p * (RT + DR_PAD);
+        float w[DR_C], y[DR_C], u[DR_C];
+#pragma unroll
+        for (int t = 0; t < DR_C; ++t) {
+          w[t] = 0.f;
+          y[t] = 0.f;
+          if (t < n) {
+            const float4* k4 = reinterpret_cast<const float4*>(kbase + t * KS);
+            const float4* q4 = reinterpret_cast<const float4*>(qbase + t * KS);
+            float w1 = 0.f, y1 = 0.f;
+#pragma unroll
+            for (int r = 0; r < RT / 4; ++r) {
+              const float4 kv = k4[r], qv = q4[r];
+              w[t] = fmaf(S[4 * r], kv.x, w[t]);
+              w1 = fmaf(S[4 * r + 1], kv.y, w1);
+              w[t] = fmaf(S[4 * r + 2], kv.z, w[t]);
+              w1 = fmaf(S[4 * r + 3], kv.w, w1);
+              y[t] = fmaf(S[4 * r], qv.x, y[t]);
+              y1 = fmaf(S[4 * r + 1], qv.y, y1);
+              y[t] = fmaf(S[4 * r + 2], qv.z, y[t]);
+              y1 = fmaf(S[4 * r + 3], qv.w, y1);
+            }
+            w[t] += w1;
+            y[t] += y1;
+          }
+        }
+        for (int off = P >> 1; off > 0; off >>= 1) {
+#pragma unroll
+          for (int t = 0; t < DR_C; ++t) {
+            w[t] += __shfl_xor(w[t], off, PYLON_WAVE);
+            y[t] += __shfl_xor(y[t], off, PYLON_WAVE);
+          }
+        }
+#pragma unroll
+        for (int t = 0; t < DR_C; ++t) {
+          u[t] = 0.f;
+          if (t < n) {
+            const float gt = gcum[t];
+            float acc = vs[t * vg + j] - gt * w[t];
+            float o = gt * y[t];
+            // row t of both matrices in 16-byte pieces, fetched before the chain that uses them
+            float ar[DR_C], br[DR_C];
+#pragma unroll
+            for (int c = 0; c <= t / 4; ++c) {
+              const float4 av = *reinterpret_cast<const float4*>(amat + t * DR_C + 4 * c);
+              const float4 bv = *reinterpret_cast<const float4*>(bmat + t * DR_C + 4 * c);
+              ar[4 * c] = av.x, ar[4 * c + 1] = av.y, ar[4 * c + 2] = av.z, ar[4 * c + 3] = av.w;
+              br[4 * c] = bv.x, br[4 * c + 1] = bv.y, br[4 * c + 2] = bv.z, br[4 * c + 3] = bv.w;
+            }
+#pragma unroll
+            for (int sx = 0; sx < t; ++sx) {
+              acc = fmaf(-ar[sx], u[sx], acc);
+              o = fmaf(br[sx], u[sx], o);
+            }
+            u[t] = betas[t] * acc;
+            o = fmaf(br[t], u[t], o);
+            if (p == 0) os[t * vg + j] = o;
+          }
+        }
+        const float gn = gcum[n - 1];
+#pragma unroll
+        for (int r = 0; r < RT; ++r) S[r] *= gn;
+#pragma unroll
+        for (int t = 0; t < DR_C; ++t) {
+          if (t < n) {
+            const float c = gend[t] * u[t];
+            const float4* k4 = reinterpret_cast<const float4*>(kbase + t * KS);
+#pragma unroll
+            for (int r = 0; r < RT / 4; ++r) {
+              const float4 kv = k4[r];
+              S[4 * r] = fmaf(kv.x, c, S[4 * r]);
+              S[4 * r + 1] = fmaf(kv.y, c, S[4 * r + 1]);
+              S[4 * r + 2] = fmaf(kv.z, c, S[4 * r + 2]);
+              S[4 * r + 3] = fmaf(kv.w, c, S[4 * r + 3]);
+            }
+          }
+        }
+      }
+    } else
     if (owner) {  // the P threads of a column are all here or all away
       for (int i = 0; i < n; ++i) {
         const float4* k4 = reinterpret_cast<const float4*>(ks + i * KS + p * (RT + DR_PAD));
         const float4* q4 = reinterpret_cast<const float4*>(qs + i * KS + p * (RT + DR_PAD));
-        float a = 0.f;
+        // four chains of additions each, so that a sum does not wait for itself
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
 #pragma unroll
         for (int r = 0; r < RT / 4; ++r) {
           const float4 v = k4[r];
-          a = fmaf(S[4 * r], v.x, a);
-          a = fmaf(S[4 * r + 1], v.y, a);
-          a = fmaf(S[4 * r + 2], v.z, a);
-          a = fmaf(S[4 * r + 3], v.w, a);
+          a0 = fmaf(S[4 * r], v.x, a0);
+          a1 = fmaf(S[4 * r + 1], v.y, a1);
+          a2 = fmaf(S[4 * r + 2], v.z, a2);
+          a3 = fmaf(S[4 * r + 3], v.w, a3);
         }
+        float a = (a0 + a1) + (a2 + a3);
         for (int off = P >> 1; off > 0; off >>= 1) a += __shfl_xor(a, off, PYLON_WAVE);
         const float g = decays[i];
         const float u = betas[i] * (vs[i * vg + j] - g * a);
-        float o = 0.f;
+        float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
         for (int r = 0; r < RT / 4; ++r) {
           const float4 v = q4[r], w = k4[r];  // the keys once more from LDS: cheaper than holding them
-          const float qq[4] = {v.x, v.y, v.z, v.w}, kk[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            S[4 * r + c] = fmaf(kk[c], u, g * S[4 * r + c]);
-            o = fmaf(S[4 * r + c], qq[c], o);
-          }
+          S[4 * r] = fmaf(w.x, u, g * S[4 * r]);
+          S[4 * r + 1] = fmaf(w.y, u, g * S[4 * r + 1]);
+          S[4 * r + 2] = fmaf(w.z, u, g * S[4 * r + 2]);
+          S[4 * r + 3] = fmaf(w.w, u, g * S[4 * r + 3]);
+          o0 = fmaf(S[4 * r], v.x, o0);
+          o1 = fmaf(S[4 * r + 1], v.y, o1);
+          o2 = fmaf(S[4 * r + 2], v.z, o2);
+          o3 = fmaf(S[4 * r + 3], v.w, o3);
         }
+        float o = (o0 + o1) + (o2 + o3);
         for (int off = P >> 1; off > 0; off >>= 1) o += __shfl_xor(o, off, PYLON_WAVE);
         if (p == 0) os[i * vg + j] = o;
       }
@@ -179,11 +371,18 @@ delta_rule_finish_kernel(TO* __restrict__ out, long long out_stride, const float
 
 // How a head of dim x vdim is laid over a workgroup: P threads a column (a power of two of at most
 // 64), R elements a thread.  Returns 0 if no layout fits.
-static int delta_rule_layout(int dim, int vdim, int* P_out, int* R_out) {
+static int delta_rule_layout(int dim, int vdim, int wide, int* P_out, int* R_out) {
   int P = 1;
-  while (P * 2 <= 64 && P * 2 <= dim && vdim * P * 2 <= 256) P *= 2;
+  if (wide) {
+    // the chunked form: as many threads a column as fill a workgroup of 256, short slices
+    while (P * 2 <= 64 && P * 2 <= dim && vdim * P * 2 <= 256) P *= 2;
+  } else {
+    // token by token: up to four threads a column while a thread's slice is longer than 32 elements (the
+    // sums over a column then end inside a quad of lanes)
+    while (P < 4 && P * 2 <= dim && (dim + P - 1) / P > 32 && vdim * P * 2 <= 1024) P *= 2;
+  }
   int R = (dim + P - 1) / P;
-  while (R > 64 && P * 2 <= 64 && vdim * P * 2 <= 1024) {
+  while (R > 64 && P * 2 <= 64 && vdim * P * 2 <= 1024) {  // more threads a column where the registers ask for it
     P *= 2;
     R = (dim + P - 1) / P;
   }
@@ -201,13 +400,14 @@ static int delta_rule_layout(int dim, int vdim, int* P_out, int* R_out) {
 // [vdim].  state: float [slots, heads, vdim, dim].  row_start: [rows + 1] prefix sums of the rows'
 // token counts; row_slots: [rows] the rows' state slots (the host guarantees they are in range).
 // col_groups > 1: a head's columns are dealt to that many workgroups, and raw (float [tokens, heads *
-// vdim]) takes o before its norm; tokens: the rows of out.
+// vdim]) takes o before its norm; tokens: the rows of out.  chunked 1: sixteen tokens at a time where
+// the sizes allow (same results up to the order of additions), else token by token.
 extern "C" int pylon_delta_rule(void* out, int out_dtype, long long out_stride, const float* qkv, long long qkv_stride,
                                 int q_off, int k_off, int v_off, const float* proj, long long proj_stride, int g_off,
                                 int b_off, int a_off, const float* a_log, const float* dt_bias, const float* norm_w,
                                 float* state, const int* row_start, const int* row_slots, int rows, int heads,
                                 int kv_heads, int dim, int vdim, float eps, float unit_eps, float q_scale,
-                                int col_groups, float* raw, int tokens, hipStream_t stream) {
+                                int col_groups, float* raw, int tokens, int chunked, hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(out_dtype), "delta_rule: unknown dtype");
   PYLON_REQUIRE(rows >= 0 && heads >= 1 && kv_heads >= 1 && heads % kv_heads == 0 && dim >= 1 && vdim >= 1,
                 "delta_rule: %d heads over %d q/k heads of %d x %d", heads, kv_heads, dim, vdim);
@@ -218,31 +418,57 @@ extern "C" int pylon_delta_rule(void* out, int out_dtype, long long out_stride, 
   PYLON_REQUIRE(col_groups >= 1 && vdim % col_groups == 0, "delta_rule: %d columns in %d groups", vdim, col_groups);
   PYLON_REQUIRE((col_groups == 1) == (raw == nullptr), "delta_rule: columns dealt to several workgroups need the buffer for o");
   const int vg = vdim / col_groups;
-  int P = 0, R = 0;
-  PYLON_REQUIRE(delta_rule_layout(dim, vg, &P, &R), "delta_rule: heads of %d x %d do not fit a workgroup", dim, vg);
+  int P = 0, R = 0, RT = 4;
+  // the chunked form where its layout fits 256 threads, slices of at most 32 elements and LDS
+  if (chunked) {
+    chunked = 0;
+    if (delta_rule_layout(dim, vg, 1, &P, &R) && R <= 32 && vg * P <= 256) {
+      while (RT < R) RT *= 2;
+      chunked = sizeof(float) * (DR_C * (2 * P * (RT + DR_PAD) + 2 * vg + 2) + 2 * DR_C * DR_C + 2 * DR_C) <= 64 * 1024;
+    }
+  }
+  // token by token: columns dealt to several workgroups take the wide layout too (measured: 10 heads of
+  // 128 x 128 over 2,048 tokens, 16 columns and 16 threads a column 1.74 ms, 64 columns and 4 threads 2.24)
+  if (!chunked)
+    PYLON_REQUIRE(delta_rule_layout(dim, vg, col_groups > 1 ? 1 : 0, &P, &R),
+                  "delta_rule: heads of %d x %d do not fit a workgroup", dim, vg);
   if (rows == 0) return 0;
-  int RT = 4;
+  RT = 4;
   while (RT < R) RT *= 2;
   const int KS = P * (RT + DR_PAD);
   const int per_token = 2 * KS + 2 * vg + 2;
-  int CT = 12000 / per_token;
+  int CT = chunked ? DR_C : 12000 / per_token;
   if (CT > 16) CT = 16;
   if (CT < 1) CT = 1;
-  const size_t lds = sizeof(float) * static_cast<size_t>(CT) * per_token;
-  PYLON_REQUIRE(lds <= 64 * 1024, "delta_rule: a token of %d x %d does not fit LDS", dim, vdim);
+  PYLON_REQUIRE(sizeof(float) * per_token <= 64 * 1024, "delta_rule: a token of %d x %d does not fit LDS", dim, vdim);
   const int threads = (vg * P + PYLON_WAVE - 1) / PYLON_WAVE * PYLON_WAVE;
+  // threads that prepare one token of a piece: a power of two, all CT tokens at once
+  if (CT > threads) CT = threads;
+  int tpt = 1;
+  while (tpt * 2 <= PYLON_WAVE && tpt * 2 * CT <= threads) tpt *= 2;
   PYLON_REQUIRE(static_cast<long long>(rows) * heads * col_groups < (1ll << 31), "delta_rule: too many rows");
+  const size_t lds = sizeof(float) * (static_cast<size_t>(CT) * per_token + 2 * DR_C * DR_C + 2 * DR_C);
   dim3 grid(static_cast<unsigned>(rows * heads * col_groups)), block(threads);
 #define GO(RTV, MAXT, TO)                                                                                     \
-  hipLaunchKernelGGL((delta_rule_kernel<RTV, MAXT, TO>), grid, block, lds, stream, (TO*)out, out_stride, qkv,   \
+  GOC(RTV, MAXT, false, TO)
+#define GOC(RTV, MAXT, CH, TO)                                                                                \
+  hipLaunchKernelGGL((delta_rule_kernel<RTV, MAXT, CH, TO>), grid, block, lds, stream, (TO*)out, out_stride, qkv, \
                      qkv_stride, q_off, k_off, v_off, proj, proj_stride, g_off, b_off, a_off, a_log, dt_bias,   \
                      norm_w, state, row_start, row_slots, heads, kv_heads, dim, vdim, P, R, CT, eps, unit_eps,  \
-                     q_scale, col_groups, raw)
+                     q_scale, col_groups, raw, tpt)
   // up to 256 threads a workgroup may use all registers of a lane; more threads share them
 #define BOTH(RTV, TO)                     \
   if (threads <= 256) GO(RTV, 256, TO);   \
   else GO(RTV, 1024, TO)
 #define PICK(TO)                         \
+  if (chunked) {                         \
+    switch (RT) {                        \
+      case 4: GOC(4, 256, true, TO); break;   \
+      case 8: GOC(8, 256, true, TO); break;   \
+      case 16: GOC(16, 256, true, TO); break; \
+      default: GOC(32, 256, true, TO); break; \
+    }                                    \
+  } else                                 \
   switch (RT) {                          \
     case 4: BOTH(4, TO); break;          \
     case 8: BOTH(8, TO); break;          \
@@ -258,6 +484,7 @@ extern "C" int pylon_delta_rule(void* out, int out_dtype, long long out_stride, 
   }
 #undef PICK
 #undef BOTH
+#undef GOC
 #undef GO
   if (raw != nullptr && tokens > 0) {
     const long long items = static_cast<long long>(tokens) * heads;

@@ -69,7 +69,7 @@ _SIGNATURES = {
     "pylon_grouped_down": [P, P, L, P, L, P, I, I, I, I, P],
     "pylon_sigmoid_gate": [P, I, P, L, L, I, I, P],
     "pylon_scaled_sum": [P, P, I, I, F, P, I, I, F, L, P],
-    "pylon_delta_rule": [P, I, L, P, L, I, I, I, P, L, I, I, I, P, P, P, P, P, P, I, I, I, I, I, F, F, F, I, P, I, P],
+    "pylon_delta_rule": [P, I, L, P, L, I, I, I, P, L, I, I, I, P, P, P, P, P, P, I, I, I, I, I, F, F, F, I, P, I, I, P],
     "pylon_expert_combine": [P, P, P, P, P, P, I, I, I, P, P, L, P, P],
 }
 

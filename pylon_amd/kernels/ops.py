@@ -678,30 +678,44 @@ def scaled_sum(a: torch.Tensor, a_scale: float, b: torch.Tensor, b_scale: float)
     return out
 
 
-def delta_rule_ok(dim: int, vdim: int) -> bool:
-    """Whether :func:`delta_rule` has a layout for heads of ``dim x vdim`` (the kernel's own rule)."""
+def _delta_rule_layout(dim: int, vdim: int, wide: bool):
+    """``(threads a column, elements a thread)`` as the kernel lays a head over a workgroup, or None."""
     p = 1
-    while p * 2 <= 64 and p * 2 <= dim and vdim * p * 2 <= 256:
-        p *= 2
+    if wide:
+        while p * 2 <= 64 and p * 2 <= dim and vdim * p * 2 <= 256:
+            p *= 2
+    else:
+        while p < 4 and p * 2 <= dim and -(-dim // p) > 32 and vdim * p * 2 <= 1024:
+            p *= 2
     r = -(-dim // p)
     while r > 64 and p * 2 <= 64 and vdim * p * 2 <= 1024:
         p *= 2
         r = -(-dim // p)
-    return dim >= 1 and vdim >= 1 and r <= 128 and vdim * p <= 1024 and (r <= 64 or vdim * p <= 256)
+    if dim < 1 or vdim < 1 or r > 128 or vdim * p > 1024 or (r > 64 and vdim * p > 256):
+        return None
+    return p, r
+
+
+def delta_rule_ok(dim: int, vdim: int, col_groups: int = 1) -> bool:
+    """Whether :func:`delta_rule` has a layout for heads of ``dim x vdim`` whose columns are dealt to
+    ``col_groups`` workgroups (the kernel's own rule)."""
+    if col_groups < 1 or vdim % col_groups:
+        return False
+    return _delta_rule_layout(dim, vdim // col_groups, col_groups > 1) is not None
 
 
 def delta_rule_col_groups(rows: int, heads: int, dim: int, vdim: int, max_count: Optional[int],
                           units: Optional[int] = None) -> int:
     """Over how many workgroups the columns of a head's state are dealt: one for steps of short rows
     (one launch, the norm inside); for rows of 64 tokens and more a power of two of at most 16 that
-    divides ``vdim``, leaves every workgroup at least 8 columns and does not start more workgroups
+    divides ``vdim``, leaves every workgroup at least 16 columns and does not start more workgroups
     than twice the compute units."""
     if max_count is None or max_count < 64:
         return 1
     units = units or _lib.compute_units()
     groups = 1
-    while (groups < 16 and vdim % (groups * 2) == 0 and vdim // (groups * 2) >= 8
-           and rows * heads * groups * 2 <= 2 * units and delta_rule_ok(dim, vdim // (groups * 2))):
+    while (groups < 16 and vdim % (groups * 2) == 0 and vdim // (groups * 2) >= 16
+           and rows * heads * groups * 2 <= 2 * units and delta_rule_ok(dim, vdim, groups * 2)):
         groups *= 2
     return groups
 
@@ -710,7 +724,8 @@ def delta_rule(qkv: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, a_log
                dt_bias: torch.Tensor, norm_weight: torch.Tensor, row_start: torch.Tensor, row_slots: torch.Tensor, *,
                rows: int, heads: int, kv_heads: int, dim: int, vdim: int, gate_off: int, beta_off: int,
                decay_off: int, eps: float, unit_eps: float, q_scale: float, out_dtype: torch.dtype,
-               max_count: Optional[int] = None, col_groups: Optional[int] = None) -> torch.Tensor:
+               max_count: Optional[int] = None, col_groups: Optional[int] = None,
+               chunked: Optional[bool] = None) -> torch.Tensor:
     """The gated delta rule over the rows of a step: per request and head ``S <- g S; u = beta (v -
     S^T k); S <- S + k u^T; o = S^T q``.  ``qkv`` float32 ``[tokens, 2 kv_heads dim + heads vdim]``
     holds q, k and v (after their convolution and activation); q and k become unit vectors per head
@@ -721,7 +736,9 @@ def delta_rule(qkv: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, a_log
     is read and left up to date.  Returns ``o / rms(o) * norm_weight * silu(gate)`` as ``[tokens,
     heads * vdim]``.  ``max_count`` (the most tokens a row brings) lets long rows have the columns of
     a head's state dealt to several workgroups (:func:`delta_rule_col_groups`; ``col_groups`` says
-    it outright); the results are the same numbers either way."""
+    it outright); the results are the same numbers either way.  ``chunked``: sixteen tokens at a
+    time, the rule written out over the piece, where the sizes allow; the same results up to the
+    order of additions (measured no faster than token by token, and not the default)."""
     if qkv.dim() != 2 or proj.dim() != 2 or qkv.dtype != torch.float32 or proj.dtype != torch.float32 \
             or qkv.stride(1) != 1 or proj.stride(1) != 1 or qkv.shape[0] != proj.shape[0]:
         raise KernelError("delta_rule takes float32 rows of q, k, v and of the projection, one per token")
@@ -744,7 +761,7 @@ def delta_rule(qkv: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, a_log
     out = torch.empty((tokens, heads * vdim), dtype=out_dtype, device=qkv.device)
     if col_groups is None:
         col_groups = delta_rule_col_groups(rows, heads, dim, vdim, max_count)
-    if col_groups < 1 or vdim % col_groups or not delta_rule_ok(dim, vdim // col_groups):
+    if not delta_rule_ok(dim, vdim, col_groups):
         raise KernelError(f"delta_rule: {vdim} columns cannot be dealt to {col_groups} workgroups")
     raw = torch.empty((tokens, heads * vdim), dtype=torch.float32, device=qkv.device) if col_groups > 1 else None
     _lib.call("pylon_delta_rule", _dev(out, "out"), dtype_code(out_dtype), heads * vdim, qkv.data_ptr(),
@@ -754,7 +771,7 @@ def delta_rule(qkv: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, a_log
               _dev(norm_weight, "norm_weight", torch.float32), _dev(state, "state", torch.float32),
               _dev(row_start, "row_start", torch.int32), _dev(row_slots, "row_slots", torch.int32), rows, heads,
               kv_heads, dim, vdim, float(eps), float(unit_eps), float(q_scale), int(col_groups), _dev(raw, "raw"),
-              tokens, _stream())
+              tokens, 1 if chunked else 0, _stream())
     return out
 
 

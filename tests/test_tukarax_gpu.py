@@ -117,7 +117,8 @@ def test_delta_rule_in_portions_of_two_requests_over_reused_slots(ops, heads, kv
                              dev(norm_w), i32(starts), i32(slots[r] for r in rows), rows=len(rows), heads=heads,
                              kv_heads=kv_heads, dim=dim, vdim=vdim, gate_off=pad, beta_off=pad + vv,
                              decay_off=pad + vv + heads, eps=eps, unit_eps=1e-6, q_scale=dim ** -0.5, out_dtype=out_dtype,
-                             col_groups=groups if len(step) % 2 else 1)  # the two ways in turns over one state
+                             col_groups=groups if len(step) % 2 else 1,  # the two ways in turns over one state,
+                             chunked=pos["x"] % 2 == 0)                  # and sixteen tokens at a time or one
         out = out.float().cpu().numpy()
         for i, rid in enumerate(rows):
             got[rid].append(out[starts[i]: starts[i + 1]])
@@ -145,9 +146,11 @@ def test_delta_rule_keeps_what_it_wrote_far_back(ops):
                 unit_eps=1e-6, q_scale=1.0, out_dtype=torch.float32)
     want = values[3] / np.sqrt((values[3] ** 2).mean() + 1e-6) * 30.0
     state = torch.zeros((1, 1, vdim, dim), device=DEV)
-    out = ops.delta_rule(dev(qkv), dev(proj), state, dev([0.0]), dev([0.0]), dev(np.ones(vdim)), i32([0, n]), i32([0]),
-                         rows=1, **args)
-    close(out[-1].cpu().numpy(), want, 1e-4, "whole")
+    for chunked in (False, True):
+        state.zero_()
+        out = ops.delta_rule(dev(qkv), dev(proj), state, dev([0.0]), dev([0.0]), dev(np.ones(vdim)), i32([0, n]), i32([0]),
+                             rows=1, chunked=chunked, **args)
+        close(out[-1].cpu().numpy(), want, 1e-4, f"whole, chunked {chunked}")
     state.zero_()
     for t in range(n):
         out = ops.delta_rule(dev(qkv[t: t + 1]), dev(proj[t: t + 1]), state, dev([0.0]), dev([0.0]), dev(np.ones(vdim)),
