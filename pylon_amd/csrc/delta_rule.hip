@@ -28,6 +28,23 @@
 #define DR_PAD 4   // floats between two slices of q or k in LDS (keeps the slices' reads off one bank)
 #define DR_HOLD 8  // elements of q, of k and of v that a thread may hold of the next piece
 
+// The sum of v over the P lanes of a column (P a power of two; the lanes j * P .. j * P + P - 1 lie
+// side by side), in every one of them.  Up to sixteen lanes it goes through the lanes' own
+// data paths (quads swapped, halves of eight mirrored, the row of sixteen mirrored): no trip to LDS,
+// which a wave alone on its SIMD would wait out; beyond that rows exchange through it.
+template <int CTRL>
+__device__ __forceinline__ float dr_moved(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float column_sum(float v, int P) {
+  if (P >= 2) v += dr_moved<0xB1>(v);   // quad_perm [1, 0, 3, 2]
+  if (P >= 4) v += dr_moved<0x4E>(v);   // quad_perm [2, 3, 0, 1]
+  if (P >= 8) v += dr_moved<0x141>(v);  // row_half_mirror
+  if (P >= 16) v += dr_moved<0x140>(v); // row_mirror
+  for (int off = 16; off < P; off <<= 1) v += __shfl_xor(v, off, PYLON_WAVE);
+  return v;
+}
+
 #define DR_C 16  // tokens of a piece in the chunked form
 
 template <int RT, int MAXT, bool CHUNK, typename TO>
@@ -225,12 +242,10 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
             y[t] += y1;
           }
         }
-        for (int off = P >> 1; off > 0; off >>= 1) {
 #pragma unroll
-          for (int t = 0; t < DR_C; ++t) {
-            w[t] += __shfl_xor(w[t], off, PYLON_WAVE);
-            y[t] += __shfl_xor(y[t], off, PYLON_WAVE);
-          }
+        for (int t = 0; t < DR_C; ++t) {
+          w[t] = column_sum(w[t], P);
+          y[t] = column_sum(y[t], P);
         }
 #pragma unroll
         for (int t = 0; t < DR_C; ++t) {
@@ -279,6 +294,56 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
       }
     } else
     if (owner) {  // the P threads of a column are all here or all away
+      if constexpr (RT <= 16) {
+        // short slices: the next token's keys, queries and numbers leave LDS while this token's chain runs
+        const float* kb = ks + p * (RT + DR_PAD);
+        const float* qb = qs + p * (RT + DR_PAD);
+        float4 kn[RT / 4], qn[RT / 4];
+        float gn = decays[0], bn = betas[0], vn = vs[j];
+#pragma unroll
+        for (int r = 0; r < RT / 4; ++r) {
+          kn[r] = reinterpret_cast<const float4*>(kb)[r];
+          qn[r] = reinterpret_cast<const float4*>(qb)[r];
+        }
+        for (int i = 0; i < n; ++i) {
+          float4 kc[RT / 4], qc[RT / 4];
+#pragma unroll
+          for (int r = 0; r < RT / 4; ++r) kc[r] = kn[r], qc[r] = qn[r];
+          const float g = gn, b = bn, v = vn;
+          if (i + 1 < n) {
+#pragma unroll
+            for (int r = 0; r < RT / 4; ++r) {
+              kn[r] = reinterpret_cast<const float4*>(kb + (i + 1) * KS)[r];
+              qn[r] = reinterpret_cast<const float4*>(qb + (i + 1) * KS)[r];
+            }
+            gn = decays[i + 1], bn = betas[i + 1], vn = vs[(i + 1) * vg + j];
+          }
+          float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+          for (int r = 0; r < RT / 4; ++r) {
+            a0 = fmaf(S[4 * r], kc[r].x, a0);
+            a1 = fmaf(S[4 * r + 1], kc[r].y, a1);
+            a2 = fmaf(S[4 * r + 2], kc[r].z, a2);
+            a3 = fmaf(S[4 * r + 3], kc[r].w, a3);
+          }
+          const float a = column_sum((a0 + a1) + (a2 + a3), P);
+          const float u = b * (v - g * a);
+          float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+#pragma unroll
+          for (int r = 0; r < RT / 4; ++r) {
+            S[4 * r] = fmaf(kc[r].x, u, g * S[4 * r]);
+            S[4 * r + 1] = fmaf(kc[r].y, u, g * S[4 * r + 1]);
+            S[4 * r + 2] = fmaf(kc[r].z, u, g * S[4 * r + 2]);
+            S[4 * r + 3] = fmaf(kc[r].w, u, g * S[4 * r + 3]);
+            o0 = fmaf(S[4 * r], qc[r].x, o0);
+            o1 = fmaf(S[4 * r + 1], qc[r].y, o1);
+            o2 = fmaf(S[4 * r + 2], qc[r].z, o2);
+            o3 = fmaf(S[4 * r + 3], qc[r].w, o3);
+          }
+          const float o = column_sum((o0 + o1) + (o2 + o3), P);
+          if (p == 0) os[i * vg + j] = o;
+        }
+      } else {
       for (int i = 0; i < n; ++i) {
         const float4* k4 = reinterpret_cast<const float4*>(ks + i * KS + p * (RT + DR_PAD));
         const float4* q4 = reinterpret_cast<const float4*>(qs + i * KS + p * (RT + DR_PAD));
@@ -292,8 +357,7 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
           a2 = fmaf(S[4 * r + 2], v.z, a2);
           a3 = fmaf(S[4 * r + 3], v.w, a3);
         }
-        float a = (a0 + a1) + (a2 + a3);
-        for (int off = P >> 1; off > 0; off >>= 1) a += __shfl_xor(a, off, PYLON_WAVE);
+        const float a = column_sum((a0 + a1) + (a2 + a3), P);
         const float g = decays[i];
         const float u = betas[i] * (vs[i * vg + j] - g * a);
         float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
@@ -309,9 +373,9 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
           o2 = fmaf(S[4 * r + 2], v.z, o2);
           o3 = fmaf(S[4 * r + 3], v.w, o3);
         }
-        float o = (o0 + o1) + (o2 + o3);
-        for (int off = P >> 1; off > 0; off >>= 1) o += __shfl_xor(o, off, PYLON_WAVE);
+        const float o = column_sum((o0 + o1) + (o2 + o3), P);
         if (p == 0) os[i * vg + j] = o;
+      }
       }
     }
     __syncthreads();
@@ -374,8 +438,8 @@ delta_rule_finish_kernel(TO* __restrict__ out, long long out_stride, const float
 static int delta_rule_layout(int dim, int vdim, int wide, int* P_out, int* R_out) {
   int P = 1;
   if (wide) {
-    // the chunked form: as many threads a column as fill a workgroup of 256, short slices
-    while (P * 2 <= 64 && P * 2 <= dim && vdim * P * 2 <= 256) P *= 2;
+    // as many threads a column (up to the sixteen of a row of lanes) as fill a workgroup of 256: short slices
+    while (P * 2 <= 16 && P * 2 <= dim && vdim * P * 2 <= 256) P *= 2;
   } else {
     // token by token: up to four threads a column while a thread's slice is longer than 32 elements (the
     // sums over a column then end inside a quad of lanes)

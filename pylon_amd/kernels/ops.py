@@ -682,7 +682,7 @@ def _delta_rule_layout(dim: int, vdim: int, wide: bool):
     """``(threads a column, elements a thread)`` as the kernel lays a head over a workgroup, or None."""
     p = 1
     if wide:
-        while p * 2 <= 64 and p * 2 <= dim and vdim * p * 2 <= 256:
+        while p * 2 <= 16 and p * 2 <= dim and vdim * p * 2 <= 256:
             p *= 2
     else:
         while p < 4 and p * 2 <= dim and -(-dim // p) > 32 and vdim * p * 2 <= 1024:
