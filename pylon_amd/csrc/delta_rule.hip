@@ -3,6 +3,9 @@
 //
 //   S <- g_t S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t
 //
+// (the kernel forms the read-out as g_t S_(t-1)^T q_t + u (k_t . q_t), the same number, so that both
+// sums over a column are taken from the state as the token finds it)
+//
 // with q and k made unit vectors per head first (x / sqrt(sum x^2 + unit_eps); q also times
 // q_scale), beta_t = sigmoid(b_t), g_t = exp(-exp(A_log) * softplus(a_t + dt_bias)) per head, and
 // every head's o_t divided by its root mean square (eps inside the root), times a weight shared by
@@ -79,6 +82,7 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
   float* bmat = amat + DR_C * DR_C; // [DR_C][DR_C]
   float* gcum = bmat + DR_C * DR_C; // [DR_C]
   float* gend = gcum + DR_C;        // [DR_C]
+  float* kqs = gend + DR_C;         // [CT <= DR_C]: the token's unit k times its scaled unit q
 
   float S[RT];
   float* st = state + ((static_cast<size_t>(row_slots[row]) * heads + h) * vdim + j0 + (owner ? j : 0)) * dim + p * R;
@@ -122,22 +126,25 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
       const float* qrow = qkv + t * qkv_stride + q_off + hk * dim;
       const float* krow = qkv + t * qkv_stride + k_off + hk * dim;
       const float* vrow = qkv + t * qkv_stride + v_off + h * vdim + j0;
-      float sq = 0.f, sk = 0.f;
+      float sq = 0.f, sk = 0.f, qk = 0.f;
       if (held) {
 #pragma unroll
         for (int e = 0; e < DR_HOLD; ++e) {
           sq = fmaf(rq[e], rq[e], sq);
           sk = fmaf(rk[e], rk[e], sk);
+          qk = fmaf(rq[e], rk[e], qk);
         }
       } else {
         for (int d = sub; d < dim; d += TPT) {
           sq = fmaf(qrow[d], qrow[d], sq);
           sk = fmaf(krow[d], krow[d], sk);
+          qk = fmaf(qrow[d], krow[d], qk);
         }
       }
       for (int off = TPT >> 1; off > 0; off >>= 1) {  // the TPT threads of a token lie side by side in one wave
         sq += __shfl_xor(sq, off, PYLON_WAVE);
         sk += __shfl_xor(sk, off, PYLON_WAVE);
+        qk += __shfl_xor(qk, off, PYLON_WAVE);
       }
       const float iq = q_scale / sqrtf(sq + unit_eps);
       const float ik = 1.0f / sqrtf(sk + unit_eps);
@@ -165,6 +172,7 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
         }
       }
       if (sub == 0) {
+        kqs[ti] = qk * iq * ik;
         betas[ti] = 1.0f / (1.0f + expf(-rb));
         const float a = ra + shift;
         const float soft = a > 20.f ? a : log1pf(expf(a));
@@ -299,7 +307,7 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
         const float* kb = ks + p * (RT + DR_PAD);
         const float* qb = qs + p * (RT + DR_PAD);
         float4 kn[RT / 4], qn[RT / 4];
-        float gn = decays[0], bn = betas[0], vn = vs[j];
+        float gn = decays[0], bn = betas[0], vn = vs[j], cn = kqs[0];
 #pragma unroll
         for (int r = 0; r < RT / 4; ++r) {
           kn[r] = reinterpret_cast<const float4*>(kb)[r];
@@ -309,72 +317,70 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
           float4 kc[RT / 4], qc[RT / 4];
 #pragma unroll
           for (int r = 0; r < RT / 4; ++r) kc[r] = kn[r], qc[r] = qn[r];
-          const float g = gn, b = bn, v = vn;
+          const float g = gn, b = bn, v = vn, kq = cn;
           if (i + 1 < n) {
 #pragma unroll
             for (int r = 0; r < RT / 4; ++r) {
               kn[r] = reinterpret_cast<const float4*>(kb + (i + 1) * KS)[r];
               qn[r] = reinterpret_cast<const float4*>(qb + (i + 1) * KS)[r];
             }
-            gn = decays[i + 1], bn = betas[i + 1], vn = vs[(i + 1) * vg + j];
+            gn = decays[i + 1], bn = betas[i + 1], vn = vs[(i + 1) * vg + j], cn = kqs[i + 1];
           }
-          float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+          // both sums over the column before the state moves: S_t^T q = g S_(t-1)^T q + u (k.q), so the
+          // read-out needs no second sum behind the update
+          float a0 = 0.f, a1 = 0.f, y0 = 0.f, y1 = 0.f;
 #pragma unroll
           for (int r = 0; r < RT / 4; ++r) {
             a0 = fmaf(S[4 * r], kc[r].x, a0);
             a1 = fmaf(S[4 * r + 1], kc[r].y, a1);
-            a2 = fmaf(S[4 * r + 2], kc[r].z, a2);
-            a3 = fmaf(S[4 * r + 3], kc[r].w, a3);
+            a0 = fmaf(S[4 * r + 2], kc[r].z, a0);
+            a1 = fmaf(S[4 * r + 3], kc[r].w, a1);
+            y0 = fmaf(S[4 * r], qc[r].x, y0);
+            y1 = fmaf(S[4 * r + 1], qc[r].y, y1);
+            y0 = fmaf(S[4 * r + 2], qc[r].z, y0);
+            y1 = fmaf(S[4 * r + 3], qc[r].w, y1);
           }
-          const float a = column_sum((a0 + a1) + (a2 + a3), P);
+          const float a = column_sum(a0 + a1, P), y = column_sum(y0 + y1, P);
           const float u = b * (v - g * a);
-          float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+          if (p == 0) os[i * vg + j] = fmaf(u, kq, g * y);
 #pragma unroll
           for (int r = 0; r < RT / 4; ++r) {
             S[4 * r] = fmaf(kc[r].x, u, g * S[4 * r]);
             S[4 * r + 1] = fmaf(kc[r].y, u, g * S[4 * r + 1]);
             S[4 * r + 2] = fmaf(kc[r].z, u, g * S[4 * r + 2]);
             S[4 * r + 3] = fmaf(kc[r].w, u, g * S[4 * r + 3]);
-            o0 = fmaf(S[4 * r], qc[r].x, o0);
-            o1 = fmaf(S[4 * r + 1], qc[r].y, o1);
-            o2 = fmaf(S[4 * r + 2], qc[r].z, o2);
-            o3 = fmaf(S[4 * r + 3], qc[r].w, o3);
           }
-          const float o = column_sum((o0 + o1) + (o2 + o3), P);
-          if (p == 0) os[i * vg + j] = o;
         }
       } else {
       for (int i = 0; i < n; ++i) {
         const float4* k4 = reinterpret_cast<const float4*>(ks + i * KS + p * (RT + DR_PAD));
         const float4* q4 = reinterpret_cast<const float4*>(qs + i * KS + p * (RT + DR_PAD));
-        // four chains of additions each, so that a sum does not wait for itself
-        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+        // chains of additions side by side, so that a sum does not wait for itself
+        float a0 = 0.f, a1 = 0.f, y0 = 0.f, y1 = 0.f;
 #pragma unroll
         for (int r = 0; r < RT / 4; ++r) {
-          const float4 v = k4[r];
-          a0 = fmaf(S[4 * r], v.x, a0);
-          a1 = fmaf(S[4 * r + 1], v.y, a1);
-          a2 = fmaf(S[4 * r + 2], v.z, a2);
-          a3 = fmaf(S[4 * r + 3], v.w, a3);
+          const float4 kv = k4[r], qv = q4[r];
+          a0 = fmaf(S[4 * r], kv.x, a0);
+          a1 = fmaf(S[4 * r + 1], kv.y, a1);
+          a0 = fmaf(S[4 * r + 2], kv.z, a0);
+          a1 = fmaf(S[4 * r + 3], kv.w, a1);
+          y0 = fmaf(S[4 * r], qv.x, y0);
+          y1 = fmaf(S[4 * r + 1], qv.y, y1);
+          y0 = fmaf(S[4 * r + 2], qv.z, y0);
+          y1 = fmaf(S[4 * r + 3], qv.w, y1);
         }
-        const float a = column_sum((a0 + a1) + (a2 + a3), P);
+        const float a = column_sum(a0 + a1, P), y = column_sum(y0 + y1, P);
         const float g = decays[i];
         const float u = betas[i] * (vs[i * vg + j] - g * a);
-        float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+        if (p == 0) os[i * vg + j] = fmaf(u, kqs[i], g * y);
 #pragma unroll
         for (int r = 0; r < RT / 4; ++r) {
-          const float4 v = q4[r], w = k4[r];  // the keys once more from LDS: cheaper than holding them
+          const float4 w = k4[r];  // the keys once more from LDS: cheaper than holding them
           S[4 * r] = fmaf(w.x, u, g * S[4 * r]);
           S[4 * r + 1] = fmaf(w.y, u, g * S[4 * r + 1]);
           S[4 * r + 2] = fmaf(w.z, u, g * S[4 * r + 2]);
           S[4 * r + 3] = fmaf(w.w, u, g * S[4 * r + 3]);
-          o0 = fmaf(S[4 * r], v.x, o0);
-          o1 = fmaf(S[4 * r + 1], v.y, o1);
-          o2 = fmaf(S[4 * r + 2], v.z, o2);
-          o3 = fmaf(S[4 * r + 3], v.w, o3);
         }
-        const float o = column_sum((o0 + o1) + (o2 + o3), P);
-        if (p == 0) os[i * vg + j] = o;
       }
       }
     }
@@ -488,7 +494,7 @@ extern "C" int pylon_delta_rule(void* out, int out_dtype, long long out_stride, 
     chunked = 0;
     if (delta_rule_layout(dim, vg, 1, &P, &R) && R <= 32 && vg * P <= 256) {
       while (RT < R) RT *= 2;
-      chunked = sizeof(float) * (DR_C * (2 * P * (RT + DR_PAD) + 2 * vg + 2) + 2 * DR_C * DR_C + 2 * DR_C) <= 64 * 1024;
+      chunked = sizeof(float) * (DR_C * (2 * P * (RT + DR_PAD) + 2 * vg + 2) + 2 * DR_C * DR_C + 3 * DR_C) <= 64 * 1024;
     }
   }
   // token by token: columns dealt to several workgroups take the wide layout too (measured: 10 heads of
@@ -511,7 +517,7 @@ extern "C" int pylon_delta_rule(void* out, int out_dtype, long long out_stride, 
   int tpt = 1;
   while (tpt * 2 <= PYLON_WAVE && tpt * 2 * CT <= threads) tpt *= 2;
   PYLON_REQUIRE(static_cast<long long>(rows) * heads * col_groups < (1ll << 31), "delta_rule: too many rows");
-  const size_t lds = sizeof(float) * (static_cast<size_t>(CT) * per_token + 2 * DR_C * DR_C + 2 * DR_C);
+  const size_t lds = sizeof(float) * (static_cast<size_t>(CT) * per_token + 2 * DR_C * DR_C + 3 * DR_C);
   dim3 grid(static_cast<unsigned>(rows * heads * col_groups)), block(threads);
 #define GO(RTV, MAXT, TO)                                                                                     \
   GOC(RTV, MAXT, false, TO)
