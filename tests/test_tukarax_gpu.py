@@ -649,6 +649,50 @@ def test_greedy_generation_through_the_engine(tmp, name, dtype, graphs, page):
             sequence.append(produced)
 
 
+@pytest.mark.parametrize("name, dtype", [("B", "float32"), ("D", "float32"), ("B", "bfloat16")])
+def test_the_replay_program_as_a_user_runs_it(tmp, tmp_path, name, dtype):
+    """``bin/trace_run`` as a subprocess over pages of 64 and four slots: up to four live requests,
+    portions of some beside single tokens of others, pages and slots used again; the logits files
+    against the plain model."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    from tests import traces
+
+    root = Path(__file__).resolve().parent.parent
+    case = Case(tmp, name, dtype, (5, 90, 64, 33, 70, 1), seed=11)
+    steps = traces.mixed(case.requests, seed=7)
+    out = tmp_path / "out"
+    proc = subprocess.Popen(
+        [sys.executable, str(root / "bin" / "trace_run"), "--model", str(case.folder), "--dtype", dtype,
+         "--out", str(out), "--max-tokens", str(traces.peak_tokens(steps))],
+        stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, cwd=str(tmp_path),
+        env=dict(os.environ, PYTHONUNBUFFERED="1"))
+    try:
+        for step in steps:
+            proc.stdin.write(json.dumps(step) + "\n")
+            proc.stdin.flush()
+            assert proc.stdout.readline().strip() == f"done {step['step']}"
+        proc.stdin.close()
+        assert proc.wait(timeout=60) == 0
+    finally:
+        if proc.poll() is None:
+            proc.kill()
+    vocab = case.cfg["vocab"]
+    outputs = {}
+    for step in steps:
+        wanted = sum(len(e["want"]) for e in step["entries"])
+        if wanted:
+            outputs[step["step"]] = np.fromfile(out / f"{step['step']}.f32", dtype="<f4").reshape(wanted, vocab)
+    got = traces.collect(steps, outputs, vocab)
+    for rid in case.requests:
+        assert len(got[rid]) == len(case.requests[rid])
+        case.check(rid, np.asarray(got[rid]), "replayed")
+
+
 def draw_config(seed: int):
     """A configuration drawn over what config.json allows: layers in any order, heads and sizes in
     steps of 8 and a few odd ones, chunks that are no multiple of anything, with and without
