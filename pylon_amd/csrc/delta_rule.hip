@@ -48,6 +48,22 @@ __device__ __forceinline__ float column_sum(float v, int P) {
   return v;
 }
 
+// The same for columns of at most sixteen lanes without a branch: all four steps are taken, and a step
+// that would reach past the column adds its neighbour times zero (`steps` holds the four factors).
+struct ColumnSteps {
+  float f1, f2, f4, f8;
+};
+__device__ __forceinline__ ColumnSteps column_steps(int P) {
+  return ColumnSteps{P >= 2 ? 1.f : 0.f, P >= 4 ? 1.f : 0.f, P >= 8 ? 1.f : 0.f, P >= 16 ? 1.f : 0.f};
+}
+__device__ __forceinline__ float column_sum(float v, const ColumnSteps& steps) {
+  v = fmaf(dr_moved<0xB1>(v), steps.f1, v);
+  v = fmaf(dr_moved<0x4E>(v), steps.f2, v);
+  v = fmaf(dr_moved<0x141>(v), steps.f4, v);
+  v = fmaf(dr_moved<0x140>(v), steps.f8, v);
+  return v;
+}
+
 #define DR_C 16  // tokens of a piece in the chunked form
 
 template <int RT, int MAXT, bool CHUNK, typename TO>
@@ -95,6 +111,7 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
   // into registers before the walk over this piece, so that their way from memory is hidden behind it.
   const int ti = tid / TPT, sub = tid - ti * TPT;
   const bool held = dim <= DR_HOLD * TPT && vg <= DR_HOLD * TPT;
+  const ColumnSteps token_steps = column_steps(TPT);
   float rq[DR_HOLD], rk[DR_HOLD], rv[DR_HOLD], rb = 0.f, ra = 0.f;
   auto fetch = [&](int c0) {
     const int n = end - c0 < CT ? end - c0 : CT;
@@ -141,10 +158,11 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
           qk = fmaf(qrow[d], krow[d], qk);
         }
       }
-      for (int off = TPT >> 1; off > 0; off >>= 1) {  // the TPT threads of a token lie side by side in one wave
-        sq += __shfl_xor(sq, off, PYLON_WAVE);
-        sk += __shfl_xor(sk, off, PYLON_WAVE);
-        qk += __shfl_xor(qk, off, PYLON_WAVE);
+      // the TPT threads of a token lie side by side in one wave
+      if (TPT <= 16) {
+        sq = column_sum(sq, token_steps), sk = column_sum(sk, token_steps), qk = column_sum(qk, token_steps);
+      } else {
+        sq = column_sum(sq, TPT), sk = column_sum(sk, TPT), qk = column_sum(qk, TPT);
       }
       const float iq = q_scale / sqrtf(sq + unit_eps);
       const float ik = 1.0f / sqrtf(sk + unit_eps);
@@ -302,7 +320,8 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
       }
     } else
     if (owner) {  // the P threads of a column are all here or all away
-      if constexpr (RT <= 16) {
+      if (RT <= 16 && P <= 16) {
+        const ColumnSteps steps = column_steps(P);
         // short slices: the next token's keys, queries and numbers leave LDS while this token's chain runs
         const float* kb = ks + p * (RT + DR_PAD);
         const float* qb = qs + p * (RT + DR_PAD);
@@ -318,13 +337,14 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
 #pragma unroll
           for (int r = 0; r < RT / 4; ++r) kc[r] = kn[r], qc[r] = qn[r];
           const float g = gn, b = bn, v = vn, kq = cn;
-          if (i + 1 < n) {
+          {
+            const int nx = i + 1 < n ? i + 1 : i;  // the last token fetches itself again: no branch
 #pragma unroll
             for (int r = 0; r < RT / 4; ++r) {
-              kn[r] = reinterpret_cast<const float4*>(kb + (i + 1) * KS)[r];
-              qn[r] = reinterpret_cast<const float4*>(qb + (i + 1) * KS)[r];
+              kn[r] = reinterpret_cast<const float4*>(kb + nx * KS)[r];
+              qn[r] = reinterpret_cast<const float4*>(qb + nx * KS)[r];
             }
-            gn = decays[i + 1], bn = betas[i + 1], vn = vs[(i + 1) * vg + j], cn = kqs[i + 1];
+            gn = decays[nx], bn = betas[nx], vn = vs[nx * vg + j], cn = kqs[nx];
           }
           // both sums over the column before the state moves: S_t^T q = g S_(t-1)^T q + u (k.q), so the
           // read-out needs no second sum behind the update
@@ -340,9 +360,9 @@ delta_rule_kernel(TO* __restrict__ out, long long out_stride, const float* __res
             y0 = fmaf(S[4 * r + 2], qc[r].z, y0);
             y1 = fmaf(S[4 * r + 3], qc[r].w, y1);
           }
-          const float a = column_sum(a0 + a1, P), y = column_sum(y0 + y1, P);
+          const float a = column_sum(a0 + a1, steps), y = column_sum(y0 + y1, steps);
           const float u = b * (v - g * a);
-          if (p == 0) os[i * vg + j] = fmaf(u, kq, g * y);
+          os[i * vg + j] = fmaf(u, kq, g * y);  // every lane of the column holds the same number
 #pragma unroll
           for (int r = 0; r < RT / 4; ++r) {
             S[4 * r] = fmaf(kc[r].x, u, g * S[4 * r]);
