@@ -533,7 +533,7 @@ def test_the_stream_after_every_layer(tmp, name, page):
 @pytest.mark.parametrize("name, dtype, page", [("A", "float32", 16), ("B", "float32", 16), ("C", "float32", 16),
                                                 ("D", "float32", 32), ("A", "bfloat16", 16), ("B", "bfloat16", 64),
                                                 ("B", "bfloat16", 32), ("C", "bfloat16", 64), ("D", "bfloat16", 64),
-                                                ("C", "float32", 64)])
+                                                ("C", "float32", 64), ("E", "float32", 64), ("E", "bfloat16", 64)])
 def test_whole_token_by_token_and_in_portions(tmp, name, dtype, page):
     """Pages of 16 tokens run the general attention kernel everywhere; with pages of 32 and 64 the
     left mixers with heads of 64 or 128 run on the matrix cores."""

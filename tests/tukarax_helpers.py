@@ -89,7 +89,17 @@ TUKARAX_D = {
                _moe(5, 2, 48)),
     ],
 }
-CONFIGS = {"A": TUKARAX_A, "B": TUKARAX_B, "C": TUKARAX_C, "D": TUKARAX_D}
+# E: nothing is a multiple of 8: a width of 100, experts of 20 hidden units, a vocabulary of 301, heads
+# of 20, 12 and 10 elements: every product and every expert path falls back to its general kernel.
+TUKARAX_E = {
+    "architecture": "Tukarax", "vocab": 301, "width": 100, "norm": {"eps": 1e-6},
+    "layers": [
+        _layer("attention", _attention(5, 5, 12, 10, 0.3, _rot(1.0e4, 6, (3.0, 20, 5.0, 1.0)), 9, 7.0), _moe(3, 2, 20)),
+        _layer("parallel", _parallel(_attention(2, 1, 20, 20, 0.2, _rot(777.0, 10)), _delta(4, 2, 10, 6, 3), 0.9, 1.1),
+               _moe(11, 5, 12)),
+    ],
+}
+CONFIGS = {"A": TUKARAX_A, "B": TUKARAX_B, "C": TUKARAX_C, "D": TUKARAX_D, "E": TUKARAX_E}
 
 
 def make_folder(tmp: Path, name: str, *, dtype: str = "float32", seed: int = 5, std: float = 0.12,
